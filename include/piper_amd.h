@@ -1,0 +1,220 @@
+/*
+ * piper_amd.h -- C ABI of libpiper_amd.so: the per-device compute of one Piper stage
+ * (MoE expert region + ZeRO bucket path) as hand-written gfx950 HIP kernels.
+ *
+ * Conventions for every entry point
+ *   - all pointers are DEVICE pointers unless the parameter is documented "host";
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *   - nothing synchronises the host, nothing allocates: scratch memory is passed
+ *     in by the caller and sized by the matching *_workspace_bytes query;
+ *   - the return value is 0 on success, a negative PK_ERR_* code for an argument
+ *     error (nothing was launched), or a positive hipError_t value;
+ *   - `dtype` arguments use the PK_F32 / PK_BF16 codes below;
+ *   - row-major, contiguous tensors; T tokens, H hidden, E experts, K top-k,
+ *     I expert intermediate size, A = T*K routed rows.
+ *
+ * The reference (github.com/uw-syfi/piper) is pure Python, so there is no FFI to
+ * mirror symbol-for-symbol; each entry point names the reference ATen sequence it
+ * replaces (file:line under the reference tree).
+ */
+#ifndef PIPER_AMD_H
+#define PIPER_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PK_OK 0
+#define PK_ERR_ARG (-1)         /* null pointer / negative size / bad enum            */
+#define PK_ERR_SHAPE (-2)       /* shape not supported by the kernels (see each call) */
+#define PK_ERR_ALIGN (-3)       /* pointer or leading dimension not 16-byte aligned   */
+#define PK_ERR_WORKSPACE (-4)   /* workspace too small                                */
+#define PK_ERR_UNSUPPORTED (-5) /* dtype / option combination not built               */
+
+#define PK_F32 0
+#define PK_BF16 1
+
+#define PK_MAX_EXPERTS 1024
+#define PK_MAX_TOPK 64
+
+
+typedef void* pk_stream_t;
+
+#define PK_API __attribute__((visibility("default")))
+
+/* Library version (major*10000 + minor*100 + patch) and a static message for a
+ * negative status code. */
+PK_API int pk_version(void);
+PK_API const char* pk_status_string(int status);
+
+/* ------------------------------------------------------------------ routing */
+
+/* logits[T,E] (f32) = x[T,H] (x_dtype) . w_gate[E,H]^T (f32) + gate_bias[E] (f32, may be NULL),
+ * fp32 accumulation.  Replaces the gate Linear inside `self.router(x, expert_bias)`
+ * (examples/models/qwen3.py:237-241; MoEArgs.gate_bias at :45). */
+PK_API int pk_gate_logits(const void* x, int x_dtype, const float* w_gate, const float* gate_bias,
+                   float* logits, int64_t T, int64_t H, int64_t E, pk_stream_t stream);
+
+/* Softmax over experts in fp32, top-K selection, optional renormalisation of the K
+ * selected scores (route_norm) and scaling (route_scale).
+ *   selection key: the fp32 logit; larger first; equal logits -> lower expert index first
+ *   (-0.0 == +0.0; NaN sorts as largest, as torch.sort does).
+ *   top_scores[T,K] f32, top_idx[T,K] i32 in selection order (best first).
+ * Replaces the softmax/top-k/renorm part of the router call (qwen3.py:237-241,
+ * score_func="softmax", route_norm/route_scale at qwen3.py:43-44,172-173).
+ * Limits: 1 <= K <= min(E, PK_MAX_TOPK), E <= PK_MAX_EXPERTS. */
+PK_API int pk_route_topk(const float* logits, int64_t T, int64_t E, int64_t K, int route_norm,
+                  float route_scale, float* top_scores, int32_t* top_idx, pk_stream_t stream);
+
+/* Backward of pk_route_topk: d_logits[T,E] (f32, fully written) from d_top_scores[T,K]. */
+PK_API int pk_route_topk_bwd(const float* logits, const int32_t* top_idx, const float* d_top_scores,
+                      int64_t T, int64_t E, int64_t K, int route_norm, float route_scale,
+                      float* d_logits, pk_stream_t stream);
+
+/* Backward of pk_gate_logits.
+ *   d_x_f32[T,H]   (f32)  = d_logits . w_gate                (written, not accumulated)
+ *   d_w_gate[E,H]  (f32) += or = d_logits^T . x              (accumulate != 0 adds)
+ *   d_gate_bias[E] (f32) += or = column sums of d_logits     (may be NULL)
+ * d_x_f32 or d_w_gate may be NULL to skip that product. */
+PK_API int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const float* w_gate,
+                       float* d_x_f32, float* d_w_gate, float* d_gate_bias, int accumulate,
+                       int64_t T, int64_t H, int64_t E, pk_stream_t stream);
+
+/* Stable counting sort of the A = T*K flat slots (slot = t*K + k) by expert id.
+ *   counts[E]   i32  tokens per expert                          (histogram)
+ *   starts[E+1] i32  exclusive prefix sum, starts[E] = A        (qwen3_bmm_experts_patch.py:27)
+ *   perm[A]     i32  sorted position -> flat slot  ("token_indices_experts_sorted")
+ *   inv_perm[A] i32  flat slot -> sorted position
+ * Within an expert, slots stay in ascending order (= torch.argsort(stable=True)).
+ * Replaces the reorderer call (qwen3.py:243-247).  Expert ids must lie in [0,E). */
+PK_API int64_t pk_sort_workspace_bytes(int64_t A, int64_t E);
+PK_API int pk_sort_by_expert(const int32_t* top_idx, int64_t A, int64_t E, int32_t* counts,
+                      int32_t* starts, int32_t* perm, int32_t* inv_perm, void* workspace,
+                      int64_t workspace_bytes, pk_stream_t stream);
+
+/* starts[E+1] (i32) from counts[E] given as int32 (counts_is_i64 == 0) or int64.
+ * For callers that hand pk_grouped_swiglu_* a `num_tokens_per_expert` tensor
+ * (qwen3_bmm_experts_patch.py:24-27). */
+PK_API int pk_counts_to_starts(const void* counts, int counts_is_i64, int64_t E, int32_t* starts,
+                        pk_stream_t stream);
+
+/* ------------------------------------------------- permute / unpermute+combine */
+
+/* routed[p,:] = x[perm[p] / K, :] for p in [0,A).   (qwen3.py:250) */
+PK_API int pk_permute_fwd(const void* x, int dtype, const int32_t* perm, void* routed, int64_t A,
+                   int64_t H, int64_t K, pk_stream_t stream);
+
+/* d_x[t,:] = sum_k d_routed[inv_perm[t*K+k], :]  (+ addend_f32[t,:] when not NULL), fp32
+ * accumulation in ascending k, rounded once to `dtype`.  Deterministic replacement for the
+ * index_put(accumulate) autograd emits for qwen3.py:250. */
+PK_API int pk_permute_bwd(const void* d_routed, int dtype, const int32_t* inv_perm,
+                   const float* addend_f32, void* d_x, int64_t T, int64_t H, int64_t K,
+                   pk_stream_t stream);
+
+/* out[t,:] = sum_k top_scores[t,k] * y_sorted[inv_perm[t*K+k], :], fp32 accumulation in
+ * ascending k, rounded once to `dtype`.  Fuses the unpermute scatter and the fp32 bmm
+ * combine (qwen3.py:265-283). */
+PK_API int pk_combine_fwd(const void* y_sorted, int dtype, const int32_t* inv_perm,
+                   const float* top_scores, void* out, int64_t T, int64_t H, int64_t K,
+                   pk_stream_t stream);
+
+/* Backward of pk_combine_fwd, per sorted row p (slot = perm[p], t = slot / K):
+ *   d_y_sorted[p,:]     = top_scores[slot] * d_out[t,:]          (dtype)
+ *   d_top_scores[slot]  = sum_h d_out[t,h] * y_sorted[p,h]       (f32) */
+PK_API int pk_combine_bwd(const void* d_out, const void* y_sorted, int dtype, const int32_t* perm,
+                   const float* top_scores, void* d_y_sorted, float* d_top_scores, int64_t A,
+                   int64_t H, int64_t K, pk_stream_t stream);
+
+/* ------------------------------------------------------ grouped SwiGLU experts
+ * Expert e owns rows [starts[e], starts[e+1]) of every [A, *] operand.
+ * Weights: w1 (gate) [E,I,H], w3 (up) [E,I,H], w2 (down) [E,H,I]
+ * (BmmExperts, qwen3_bmm_experts_patch.py:90-110).
+ * Together these replace _run_bmm_experts (qwen3_bmm_experts_patch.py:11-50) and the
+ * autograd graph torch builds for it (src/executors.py:257-296).
+ * bf16 runs on MFMA tiles and needs H % 64 == 0 and I % 64 == 0; f32 runs on a
+ * tiled FMA kernel with no shape restriction.
+ */
+
+/* Forward.  x_rows[A_x,H]: when row_map is NULL, row p of the A operand is x_rows[p]
+ * (x already expert-sorted, the reference boundary); otherwise it is
+ * x_rows[row_map[p] / row_map_div] (permute fused into the operand load; pass perm and K).
+ *   g[A,I] = x . w1[e]^T,  u[A,I] = x . w3[e]^T   (saved for backward)
+ *   h[A,I] = silu(g) * u
+ *   y[A,H] = h . w2[e]^T */
+PK_API int pk_grouped_swiglu_fwd(const void* x_rows, const int32_t* row_map, int64_t row_map_div,
+                          const void* w1, const void* w2, const void* w3,
+                          const int32_t* starts, void* g, void* u, void* h, void* y,
+                          int64_t A, int64_t H, int64_t I, int64_t E, int dtype,
+                          pk_stream_t stream);
+
+/* Input gradient (Piper's BWD_I task, src/executors.py:353-411).
+ *   d_h = d_y . w2[e];  d_g = d_h * u * silu'(g);  d_u = d_h * silu(g)   -> d_g, d_u [A,I]
+ *   d_x_sorted[A,H] = d_g . w1[e] + d_u . w3[e] */
+PK_API int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, const void* w3,
+                            const void* g, const void* u, const int32_t* starts, void* d_g,
+                            void* d_u, void* d_x_sorted, int64_t A, int64_t H, int64_t I,
+                            int64_t E, int dtype, pk_stream_t stream);
+
+/* Weight gradient (Piper's BWD_W task, src/executors.py:413-476).
+ *   d_w2[e] (+)= d_y[rows_e]^T . h[rows_e]          [H,I]
+ *   d_w1[e] (+)= d_g[rows_e]^T . x[rows_e]          [I,H]
+ *   d_w3[e] (+)= d_u[rows_e]^T . x[rows_e]          [I,H]
+ * x rows are addressed as in the forward (row_map / row_map_div).  accumulate != 0 adds
+ * to the existing contents (gradient accumulation over microbatches,
+ * src/executors.py:333-343); otherwise every element is overwritten, with zeros for
+ * an expert that received no rows. */
+PK_API int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, const void* d_u,
+                            const void* x_rows, const int32_t* row_map, int64_t row_map_div,
+                            const int32_t* starts, void* d_w1, void* d_w2, void* d_w3,
+                            int accumulate, int64_t A, int64_t H, int64_t I, int64_t E,
+                            int dtype, pk_stream_t stream);
+
+/* ------------------------------------------------------------- ZeRO bucket path */
+
+/* HOST function.  offsets[i] (in elements) of n tensors laid out back to back, each start
+ * rounded up to `align_bytes` (a power of two, multiple of elem_size; 1 reproduces the
+ * reference's unaligned running sum, src/actor.py:545-554).  Returns the padded total
+ * (also a multiple of the alignment), or a negative PK_ERR_*.  numels/offsets: host. */
+PK_API int64_t pk_bucket_plan(const int64_t* numels, int64_t n, int64_t elem_size,
+                       int64_t align_bytes, int64_t* offsets);
+
+/* Multi-tensor copy/cast/accumulate into a flat bucket, one launch per
+ * 120 tensors (more are split over several launches):  flat[offsets[i] : offsets[i]+numels[i]] (+)= cast(src[i]).
+ *   srcs: HOST array of n device pointers (NULL entries are skipped: "grad is None");
+ *   offsets, numels: HOST arrays (elements);  src_dtype -> dst_dtype any of f32/bf16.
+ * Replaces the per-tensor `flat[o:o+n].add_(g.reshape(-1).to(f32))` loop
+ * (src/runtime.py:275-282) and the torch.cat flatten (src/actor.py:534). */
+PK_API int pk_bucket_pack(const void* const* srcs, const int64_t* offsets, const int64_t* numels,
+                   int64_t n, int src_dtype, void* flat, int dst_dtype, int accumulate,
+                   pk_stream_t stream);
+
+/* Inverse of pk_bucket_pack without accumulation: dst[i][:] = cast(flat[offsets[i] : ...]).
+ * Only needed when parameters are NOT views of the bucket (src/runtime.py:329-339 keeps
+ * them as views, in which case unflatten is free). */
+PK_API int pk_bucket_unpack(const void* flat, int flat_dtype, void* const* dsts, const int64_t* offsets,
+                     const int64_t* numels, int64_t n, int dst_dtype, pk_stream_t stream);
+
+/* flat[0:n] = 0 for an f32 bucket (src/runtime.py:223-229). */
+PK_API int pk_bucket_zero(float* flat, int64_t n, pk_stream_t stream);
+
+/* One fused AdamW step over a whole fp32 bucket, torch.optim.AdamW operation order
+ * (decoupled decay, lerp first moment, bias-corrected step):
+ *   p *= 1 - lr*wd;  m += (g-m)*(1-b1);  v = v*b2 + (1-b2)*g*g;
+ *   p -= (lr / (1-b1^step)) * m / (sqrt(v)/sqrt(1-b2^step) + eps)
+ * grad is f32 (the bucket) and is scaled by grad_scale first (1.0f = off).
+ * shadow (may be NULL): the updated p rounded to `shadow_dtype`, written in the same pass --
+ * this is the bucket the bf16 parameter views alias, so "unflatten" costs nothing.
+ * zero_grad != 0 also clears grad in the same pass.
+ * Replaces `shard_param.grad = ...; shard_optim.step()` (src/runtime.py:470-473) and
+ * `bucket.optimizer.step()` (src/executors.py:1024-1025). */
+PK_API int pk_adamw_fused(float* master, float* exp_avg, float* exp_avg_sq, float* grad, void* shadow,
+                   int shadow_dtype, int64_t n, float lr, float beta1, float beta2, float eps,
+                   float weight_decay, int64_t step, float grad_scale, int zero_grad,
+                   pk_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PIPER_AMD_H */

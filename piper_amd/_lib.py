@@ -1,0 +1,119 @@
+"""ctypes binding of libpiper_amd.so (declared in include/piper_amd.h).
+
+The library is loaded lazily on first use and never silently replaced: if it has not been
+built, or a call returns a non-zero status, a RuntimeError is raised.  This mirrors the
+reference, where every failure inside a task is a Python exception that propagates to the
+driver (e.g. the assertions in src/runtime.py:313-328).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "libpiper_amd.so"
+
+PK_F32 = 0
+PK_BF16 = 1
+
+_c_i64 = C.c_int64
+_c_int = C.c_int
+_c_f32 = C.c_float
+_p = C.c_void_p
+
+# name -> (restype, argtypes); must list every symbol declared in include/piper_amd.h
+SIGNATURES = {
+    "pk_version": (_c_int, []),
+    "pk_status_string": (C.c_char_p, [_c_int]),
+    "pk_gate_logits": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_route_topk": (_c_int, [_p, _c_i64, _c_i64, _c_i64, _c_int, _c_f32, _p, _p, _p]),
+    "pk_route_topk_bwd": (_c_int, [_p, _p, _p, _c_i64, _c_i64, _c_i64, _c_int, _c_f32, _p, _p]),
+    "pk_gate_logits_bwd": (_c_int, [_p, _p, _c_int, _p, _p, _p, _p, _c_int, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_sort_workspace_bytes": (_c_i64, [_c_i64, _c_i64]),
+    "pk_sort_by_expert": (_c_int, [_p, _c_i64, _c_i64, _p, _p, _p, _p, _p, _c_i64, _p]),
+    "pk_counts_to_starts": (_c_int, [_p, _c_int, _c_i64, _p, _p]),
+    "pk_permute_fwd": (_c_int, [_p, _c_int, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_permute_bwd": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_combine_fwd": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_combine_bwd": (_c_int, [_p, _p, _c_int, _p, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_grouped_swiglu_fwd": (_c_int, [_p, _p, _c_i64, _p, _p, _p, _p, _p, _p, _p, _p,
+                                       _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
+    "pk_grouped_swiglu_dgrad": (_c_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p,
+                                         _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
+    "pk_grouped_swiglu_wgrad": (_c_int, [_p, _p, _p, _p, _p, _p, _c_i64, _p, _p, _p, _p, _c_int,
+                                         _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
+    "pk_bucket_plan": (_c_i64, [_p, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_bucket_pack": (_c_int, [_p, _p, _p, _c_i64, _c_int, _p, _c_int, _c_int, _p]),
+    "pk_bucket_unpack": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_int, _p]),
+    "pk_bucket_zero": (_c_int, [_p, _c_i64, _p]),
+    "pk_adamw_fused": (_c_int, [_p, _p, _p, _p, _p, _c_int, _c_i64, _c_f32, _c_f32, _c_f32, _c_f32,
+                                _c_f32, _c_i64, _c_f32, _c_int, _p]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m piper_amd.build` "
+                "(there is no fallback implementation)"
+            )
+        lib = C.CDLL(str(LIB_PATH))
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(lib, name)  # AttributeError here means header and library disagree
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = lib
+    return _lib
+
+
+def is_built() -> bool:
+    return LIB_PATH.exists()
+
+
+def status_string(status: int) -> str:
+    return load().pk_status_string(int(status)).decode()
+
+
+def call(name: str, *args):
+    """Call an int-returning entry point and raise RuntimeError on a non-zero status."""
+    rc = getattr(load(), name)(*args)
+    if rc != 0:
+        raise RuntimeError(f"{name} failed with status {rc}: {status_string(rc)}")
+    return rc
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return PK_F32
+    if dtype == torch.bfloat16:
+        return PK_BF16
+    raise TypeError(f"piper_amd kernels support float32 and bfloat16, got {dtype}")
+
+
+def ptr(t: torch.Tensor | None):
+    """Device pointer of a contiguous tensor (None -> NULL)."""
+    if t is None:
+        return None
+    if not t.is_contiguous():
+        raise ValueError("piper_amd kernels need contiguous tensors")
+    return t.data_ptr()
+
+
+def current_stream(device: torch.device | None = None):
+    """The hipStream_t of torch's current stream, so kernels respect `torch.cuda.stream(...)`
+    exactly like the ATen ops they replace (src/executors.py:231-232)."""
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_gpu(t: torch.Tensor) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            "piper_amd kernels run on the GPU only; got a tensor on "
+            f"{t.device} (there is no CPU fallback)"
+        )

@@ -1,0 +1,225 @@
+"""ZeRO bucket path on one device: bucket layout, flatten, gradient packing, optimizer step,
+unflatten.  Mirrors the runtime half of the reference -- ``BucketState`` / ``ParamStorage``
+(src/runtime.py:64-99,202-495) and the flatten block of ``_load_stage`` (src/actor.py:517-601) --
+with the same method names and arguments, so an executor written against the reference drives it
+unchanged.  Differences, all from the benchmark definition: every tensor starts on a 256-byte
+boundary, the optimizer state is an fp32 master bucket, packing is one kernel launch for all
+tensors and the optimizer is one fused AdamW launch.
+
+With one GPU dp_degree is 1: the shard is the whole bucket and reduce-scatter / all-gather are
+identities, so ``reduce_scatter_grads`` aliases ``flat_grads``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Sequence
+
+import torch
+
+from . import ops
+from .optim import FusedAdamW
+
+BUCKET_ALIGN_BYTES = 256
+
+
+@dataclass
+class BucketState:
+    """Loaded runtime state of one compute bucket (field names of src/runtime.py:64-99)."""
+
+    forward_fn: Any = None
+    forward_args: list = field(default_factory=list)
+    input_idxs: list = field(default_factory=list)
+    param_idxs: list = field(default_factory=list)
+    param_names: list = field(default_factory=list)
+    optimizer: Any = None
+    trainable_param_idxs: list = field(default_factory=list)
+
+    flat_params: torch.Tensor | None = None          # param dtype; parameters are views of it
+    flat_grads: torch.Tensor | None = None           # fp32
+    shard_param: torch.Tensor | None = None
+    shard_optimizer: Any = None
+    reduce_scatter_grads: torch.Tensor | None = None
+    param_shard_info: tuple | None = None            # (shard_start, shard_size, orig_numel)
+    param_view_specs: list = field(default_factory=list)  # (param, offset, numel, shape)
+    full_params_fresh: bool = False
+
+    def weights(self) -> list:
+        return [self.forward_args[i] for i in self.param_idxs if self.forward_args[i] is not None]
+
+    def trainable_params(self) -> list:
+        return [self.forward_args[i] for i in self.trainable_param_idxs if self.forward_args[i] is not None]
+
+
+def plan_bucket(shapes: Sequence[Sequence[int]], elem_size: int, align_bytes: int = BUCKET_ALIGN_BYTES):
+    """Element offsets of the tensors inside one bucket and the padded bucket length."""
+    numels = [int(torch.Size(s).numel()) for s in shapes]
+    return ops.bucket_plan(numels, elem_size, align_bytes)
+
+
+def flatten_params(bucket: BucketState, params: Sequence[torch.nn.Parameter], *,
+                   optim_class: Callable[..., Any] | None = None, align_bytes: int = BUCKET_ALIGN_BYTES,
+                   dp_degree: int = 1, dp_rank: int = 0, grad_dtype: torch.dtype = torch.float32) -> BucketState:
+    """The ZeRO flatten of src/actor.py:532-586: copy all parameters into one flat buffer, re-point
+    each parameter at its view, allocate the fp32 gradient bucket and build the shard optimizer."""
+    if dp_degree != 1 or dp_rank != 0:
+        raise NotImplementedError("this build runs one GPU: dp_degree must be 1")
+    params = list(params)
+    if not params:
+        raise ValueError("flatten_params: empty parameter list")
+    dtype, device = params[0].dtype, params[0].device
+    if any(p.dtype != dtype or p.device != device for p in params):
+        raise ValueError("all parameters of a bucket must share dtype and device")
+    esize = params[0].element_size()
+    # offsets must be valid for the param-dtype bucket AND the fp32 buckets that share them
+    offsets, padded = ops.bucket_plan([p.numel() for p in params], esize, align_bytes)
+    orig_numel = (offsets[-1] + params[-1].numel()) if params else 0
+
+    flat_params = torch.zeros(padded, dtype=dtype, device=device)
+    ops.bucket_pack([p.detach() for p in params], offsets, flat_params, accumulate=False)
+    view_specs = []
+    for p, off in zip(params, offsets):
+        n = p.numel()
+        p.data = flat_params[off:off + n].view(p.shape)
+        p.requires_grad_(True)
+        p.grad_dtype = grad_dtype
+        view_specs.append((p, off, n, tuple(p.shape)))
+
+    shard_param = flat_params[0:padded]
+    shard_param.requires_grad_(True)
+    shard_param.grad_dtype = None  # accept the fp32 gradient bucket as .grad
+
+    bucket.flat_params = flat_params
+    bucket.flat_grads = torch.zeros(padded, dtype=grad_dtype, device=device)
+    bucket.reduce_scatter_grads = bucket.flat_grads  # dp_degree == 1: reduce-scatter is the identity
+    bucket.shard_param = shard_param
+    bucket.shard_optimizer = (optim_class or FusedAdamW)([shard_param])
+    bucket.param_shard_info = (0, padded, orig_numel)
+    bucket.param_view_specs = view_specs
+    bucket.full_params_fresh = True
+    bucket.optimizer = None
+    return bucket
+
+
+@dataclass
+class StageStore:
+    buckets: dict = field(default_factory=dict)
+    zero_managed_ubids: set = field(default_factory=set)
+    param_sharded_ubids: set = field(default_factory=set)
+    grad_sharded_ubids: set = field(default_factory=set)
+
+    def bucket(self, ubid) -> BucketState:
+        if ubid not in self.buckets:
+            raise KeyError(f"unknown bucket id {ubid!r}")
+        return self.buckets[ubid]
+
+    def get_bucket(self, ubid):
+        return self.buckets.get(ubid)
+
+
+@dataclass
+class ParamStorage:
+    """ZeRO parameter and gradient storage of one device (src/runtime.py:202-495)."""
+
+    stages: StageStore
+    grad_buffer_dtype: torch.dtype = torch.float32
+
+    def clear_param_grads(self) -> None:
+        for bucket in self.stages.buckets.values():
+            for p, *_ in bucket.param_view_specs:
+                p.grad = None
+
+    def zero_grad_buffers(self, stream: torch.cuda.Stream | None = None) -> None:
+        """src/runtime.py:223-229."""
+        with torch.cuda.stream(stream):
+            for bucket in self.stages.buckets.values():
+                if bucket.flat_grads is not None:
+                    ops.bucket_zero(bucket.flat_grads)
+                rs = bucket.reduce_scatter_grads
+                if rs is not None and rs is not bucket.flat_grads:
+                    ops.bucket_zero(rs)
+
+    def accumulate_zero_param_grads_to_flat(self, ubid, stream: torch.cuda.Stream | None = None) -> None:
+        """Gradient pack (src/runtime.py:249-282): flat[o:o+n] += grad.to(f32) for every tensor of
+        the bucket in one launch, then drop the per-tensor grads."""
+        if ubid is None or ubid not in self.stages.zero_managed_ubids:
+            return
+        bucket = self.stages.bucket(ubid)
+        specs = bucket.param_view_specs
+        if not specs:
+            return
+        with torch.cuda.stream(stream):
+            if bucket.flat_grads is None:
+                bucket.flat_grads = torch.zeros(bucket.param_shard_info[1], dtype=self.grad_buffer_dtype,
+                                                device=bucket.flat_params.device)
+                bucket.reduce_scatter_grads = bucket.flat_grads
+            by_dtype: dict = {}
+            for param, offset, numel, _shape in specs:
+                grad = param.grad
+                if grad is None:
+                    continue
+                g = grad.detach()
+                if stream is not None:
+                    g.record_stream(stream)
+                by_dtype.setdefault(g.dtype, ([], []))
+                by_dtype[g.dtype][0].append(g.reshape(-1))
+                by_dtype[g.dtype][1].append(offset)
+            for grads, offs in by_dtype.values():
+                ops.bucket_pack(grads, offs, bucket.flat_grads, accumulate=True)
+            for param, *_ in specs:
+                param.grad = None
+
+    def alloc_full_params(self, ubid) -> None:
+        """Unflatten (src/runtime.py:312-352): make every parameter a view of the flat bucket."""
+        bucket = self.stages.bucket(ubid)
+        full = bucket.flat_params
+        assert full is not None, f"alloc_full_params: missing flat_params buffer for ubid={ubid}"
+        assert bucket.param_view_specs, f"alloc_full_params: missing param_view_specs for ubid={ubid}"
+        for param, offset, numel, shape in bucket.param_view_specs:
+            if param.data_ptr() != full.data_ptr() + offset * full.element_size():
+                param.data = full[offset:offset + numel].view(shape)
+            param.requires_grad_(True)
+        bucket.full_params_fresh = True
+
+    def free_full_params(self, ubid) -> None:
+        """One device keeps the only copy of the parameters, so there is nothing to release;
+        the bucket is only marked stale (src/runtime.py:354-371)."""
+        self.stages.bucket(ubid).full_params_fresh = False
+
+    def alloc_full_grads(self, ubid, stream: torch.cuda.Stream | None = None) -> None:
+        bucket = self.stages.bucket(ubid)
+        with torch.cuda.stream(stream):
+            if bucket.flat_grads is None:
+                bucket.flat_grads = torch.zeros(bucket.param_shard_info[1], dtype=self.grad_buffer_dtype,
+                                                device=bucket.flat_params.device)
+                bucket.reduce_scatter_grads = bucket.flat_grads
+
+    def free_full_grads(self, ubid) -> None:
+        bucket = self.stages.bucket(ubid)
+        for param, *_ in bucket.param_view_specs:
+            param.grad = None
+
+    def all_gather_full_params(self, ubid, stream: torch.cuda.Stream | None = None) -> int:
+        """dp_degree == 1: the shard is the whole bucket, so the gather moves no bytes."""
+        self.alloc_full_params(ubid)
+        return 0
+
+    def has_zero_shard_optimizers(self) -> bool:
+        return any(b.shard_optimizer is not None for b in self.stages.buckets.values())
+
+    def step_zero_shard_optimizers(self, stream: torch.cuda.Stream | None = None,
+                                   reduce_scatter_events: dict | None = None) -> None:
+        """src/runtime.py:454-484: wait for the gradient events, run each bucket's optimizer on its
+        shard with the fp32 gradient bucket as .grad."""
+        if stream is not None:
+            for evt in (reduce_scatter_events or {}).values():
+                stream.wait_event(evt)
+        for bucket in self.stages.buckets.values():
+            opt = bucket.shard_optimizer
+            if opt is None or bucket.reduce_scatter_grads is None:
+                continue
+            with torch.cuda.stream(stream):
+                bucket.shard_param.grad = bucket.reduce_scatter_grads
+                opt.step()
+            bucket.shard_param.grad = None
+            for param, *_ in bucket.param_view_specs:
+                param.grad = None

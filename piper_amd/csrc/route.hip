@@ -1,0 +1,442 @@
+// Routing: gate logits, wavefront softmax/top-k (+ backward), stable counting sort by expert.
+#include "pk_common.h"
+#include "simt_gemm.h"
+
+namespace {
+
+// ------------------------------------------------------------------ top-k
+// Order-preserving map float -> uint32 (larger float -> larger uint).  -0.0 is folded into
+// +0.0 and every NaN into the positive quiet NaN so that ties and NaNs behave like
+// torch.sort(descending=True, stable=True).
+__device__ __forceinline__ uint32_t orderable(float v) {
+  v = v + 0.0f;
+  uint32_t u = __float_as_uint(v);
+  if (v != v) u = 0x7fc00000u;
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float from_orderable(uint32_t o) {
+  const uint32_t u = (o & 0x80000000u) ? (o ^ 0x80000000u) : ~o;
+  return __uint_as_float(u);
+}
+
+constexpr int kRouteThreads = 256;  // 4 waves, one token per wave
+
+// One wave per token.  Lane l owns experts l, l+64, ... (EPL of them).
+template <int EPL>
+__global__ __launch_bounds__(kRouteThreads) void route_topk_kernel(
+    const float* __restrict__ logits, int T, int E, int K, int route_norm, float route_scale,
+    float* __restrict__ top_scores, int32_t* __restrict__ top_idx) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * (kRouteThreads / 64) + wave;
+  if (t >= T) return;
+  const float* row = logits + (int64_t)t * E;
+
+  float val[EPL];
+  unsigned long long key[EPL];
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    const int e = lane + 64 * j;
+    if (e < E) {
+      val[j] = row[e];
+      key[j] = ((unsigned long long)orderable(val[j]) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)e);
+    } else {
+      val[j] = 0.f;
+      key[j] = 0ull;  // never wins: every real key has a non-zero high word
+    }
+  }
+
+  float vmax = 0.f;
+  float my_v = 0.f;
+  int my_e = 0;
+  for (int k = 0; k < K; ++k) {
+    unsigned long long best = 0ull;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) best = key[j] > best ? key[j] : best;
+    best = pk_wave_max_u64(best);
+    const uint32_t e_win = 0xffffffffu - (uint32_t)(best & 0xffffffffull);
+    const float v_win = from_orderable((uint32_t)(best >> 32));
+#pragma unroll
+    for (int j = 0; j < EPL; ++j)
+      if ((int)e_win == lane + 64 * j) key[j] = 0ull;
+    if (k == 0) vmax = v_win;
+    if (lane == k) { my_v = v_win; my_e = (int)e_win; }
+  }
+
+  float part = 0.f;
+#pragma unroll
+  for (int j = 0; j < EPL; ++j)
+    if (lane + 64 * j < E) part += expf(val[j] - vmax);
+  const float denom = pk_wave_sum(part);
+
+  float s = (lane < K) ? expf(my_v - vmax) / denom : 0.f;
+  if (route_norm) {
+    const float S = pk_wave_sum(s);
+    s = s / (S + 1e-20f);
+  }
+  s *= route_scale;
+  if (lane < K) {
+    top_scores[(int64_t)t * K + lane] = s;
+    top_idx[(int64_t)t * K + lane] = my_e;
+  }
+}
+
+template <int EPL>
+__global__ __launch_bounds__(kRouteThreads) void route_topk_bwd_kernel(
+    const float* __restrict__ logits, const int32_t* __restrict__ top_idx,
+    const float* __restrict__ d_top_scores, int T, int E, int K, int route_norm,
+    float route_scale, float* __restrict__ d_logits) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * (kRouteThreads / 64) + wave;
+  if (t >= T) return;
+  const float* row = logits + (int64_t)t * E;
+
+  float val[EPL];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    const int e = lane + 64 * j;
+    val[j] = (e < E) ? row[e] : -INFINITY;
+    mx = fmaxf(mx, val[j]);
+  }
+  mx = pk_wave_max(mx);
+  float p[EPL];
+  float part = 0.f;
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    p[j] = (lane + 64 * j < E) ? expf(val[j] - mx) : 0.f;
+    part += p[j];
+  }
+  const float denom = pk_wave_sum(part);
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) p[j] = p[j] / denom;
+
+  // lanes k < K: selected expert, its probability, incoming gradient
+  int my_e = -1;
+  float s = 0.f, dw = 0.f;
+  if (lane < K) {
+    my_e = top_idx[(int64_t)t * K + lane];
+    s = expf(row[my_e] - mx) / denom;
+    dw = d_top_scores[(int64_t)t * K + lane];
+  }
+  float ds;
+  if (route_norm) {
+    const float S = pk_wave_sum(s) + 1e-20f;
+    const float dot = pk_wave_sum(dw * s);
+    ds = route_scale * (dw / S - dot / (S * S));
+  } else {
+    ds = route_scale * dw;
+  }
+  if (lane >= K) ds = 0.f;
+  const float D = pk_wave_sum(ds * s);  // sum_j dp_j p_j
+
+  float dp[EPL];
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) dp[j] = 0.f;
+  for (int k = 0; k < K; ++k) {
+    const int ek = __shfl(my_e, k, PK_WAVE);
+    const float dsk = __shfl(ds, k, PK_WAVE);
+#pragma unroll
+    for (int j = 0; j < EPL; ++j)
+      if (lane + 64 * j == ek) dp[j] = dsk;
+  }
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    const int e = lane + 64 * j;
+    if (e < E) d_logits[(int64_t)t * E + e] = p[j] * (dp[j] - D);
+  }
+}
+
+// ------------------------------------------------------------------ counting sort
+constexpr int kSortChunk = 512;  // flat slots per chunk; one wave walks a chunk in order
+
+__global__ __launch_bounds__(64) void sort_hist_kernel(const int32_t* __restrict__ idx, int A,
+                                                       int E, int32_t* __restrict__ chunk_hist) {
+  extern __shared__ int32_t hist[];  // [E]
+  for (int e = threadIdx.x; e < E; e += 64) hist[e] = 0;
+  __syncthreads();
+  const int base = blockIdx.x * kSortChunk;
+  for (int i = threadIdx.x; i < kSortChunk; i += 64) {
+    const int s = base + i;
+    if (s < A) {
+      const int e = idx[s];
+      if ((unsigned)e < (unsigned)E) atomicAdd(&hist[e], 1);  // out-of-range ids are dropped
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 64) chunk_hist[(int64_t)blockIdx.x * E + e] = hist[e];
+}
+
+// Single block.  counts[e] = sum over chunks; starts = exclusive scan; chunk_hist[c][e] is
+// replaced by the first output position of expert e's rows coming from chunk c.
+__global__ __launch_bounds__(1024) void sort_scan_kernel(int32_t* __restrict__ chunk_hist,
+                                                         int nchunks, int E,
+                                                         int32_t* __restrict__ counts,
+                                                         int32_t* __restrict__ starts) {
+  __shared__ int32_t scan[PK_MAX_EXPERTS];
+  const int e = threadIdx.x;
+  int total = 0;
+  if (e < E) {
+    for (int c = 0; c < nchunks; ++c) {
+      const int v = chunk_hist[(int64_t)c * E + e];
+      chunk_hist[(int64_t)c * E + e] = total;
+      total += v;
+    }
+    if (counts) counts[e] = total;
+  }
+  scan[e] = (e < E) ? total : 0;
+  __syncthreads();
+  // Hillis-Steele inclusive scan over 1024 entries
+  for (int off = 1; off < 1024; off <<= 1) {
+    const int v = (e >= off) ? scan[e - off] : 0;
+    __syncthreads();
+    scan[e] += v;
+    __syncthreads();
+  }
+  const int start = scan[e] - total;  // exclusive
+  if (e < E) {
+    starts[e] = start;
+    if (e == E - 1) starts[E] = scan[e];
+    for (int c = 0; c < nchunks; ++c) chunk_hist[(int64_t)c * E + e] += start;
+  }
+}
+
+__global__ __launch_bounds__(64) void sort_scatter_kernel(const int32_t* __restrict__ idx, int A,
+                                                          int E, const int32_t* __restrict__ chunk_base,
+                                                          int32_t* __restrict__ perm,
+                                                          int32_t* __restrict__ inv_perm) {
+  extern __shared__ int32_t base[];  // [E] next free position per expert
+  const int lane = threadIdx.x;
+  for (int e = lane; e < E; e += 64) base[e] = chunk_base[(int64_t)blockIdx.x * E + e];
+  __syncthreads();
+  const int s0 = blockIdx.x * kSortChunk;
+  const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int i = 0; i < kSortChunk; i += 64) {
+    const int s = s0 + i + lane;
+    int e = (s < A) ? idx[s] : -1;
+    if ((unsigned)e >= (unsigned)E) e = -1;
+    const bool active = e >= 0;
+    // lanes holding the same expert id
+    unsigned long long same = __ballot(active);
+    for (int b = 0; b < 10; ++b) {
+      const unsigned long long bal = __ballot((e >> b) & 1);
+      same &= ((e >> b) & 1) ? bal : ~bal;
+    }
+    int pos = 0;
+    if (active) {
+      const int rank = __popcll(same & lt_mask);
+      pos = base[e] + rank;
+    }
+    __syncthreads();
+    if (active) {
+      // the last lane of each group advances the expert's cursor
+      const int top = 63 - __clzll(same);
+      if (lane == top) base[e] += __popcll(same);
+      perm[pos] = s;
+      if (inv_perm) inv_perm[s] = pos;
+    }
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(1024) void counts_to_starts_kernel(const void* __restrict__ counts,
+                                                                int is_i64, int E,
+                                                                int32_t* __restrict__ starts) {
+  __shared__ int32_t scan[PK_MAX_EXPERTS];
+  const int e = threadIdx.x;
+  int c = 0;
+  if (e < E) c = is_i64 ? (int)reinterpret_cast<const int64_t*>(counts)[e]
+                        : reinterpret_cast<const int32_t*>(counts)[e];
+  scan[e] = c;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const int v = (e >= off) ? scan[e - off] : 0;
+    __syncthreads();
+    scan[e] += v;
+    __syncthreads();
+  }
+  if (e < E) {
+    starts[e] = scan[e] - c;
+    if (e == E - 1) starts[E] = scan[e];
+  }
+}
+
+// ------------------------------------------------------------------ small helpers
+__global__ void bias_fill_kernel(float* __restrict__ logits, const float* __restrict__ bias,
+                                 int64_t T, int E) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < T * E) logits[i] = bias[i % E];
+}
+
+// d_bias[e] (+)= sum_t d_logits[t,e]; one block per expert
+__global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ d_logits, int64_t T,
+                                                     int E, float* __restrict__ d_bias,
+                                                     int accumulate) {
+  __shared__ float red[16];
+  const int e = blockIdx.x;
+  float s = 0.f;
+  for (int64_t t = threadIdx.x; t < T; t += blockDim.x) s += d_logits[t * E + e];
+  s = pk_block_sum(s, red);
+  if (threadIdx.x == 0) d_bias[e] = accumulate ? d_bias[e] + s : s;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pk_version(void) { return 100; }
+
+const char* pk_status_string(int status) {
+  switch (status) {
+    case PK_OK: return "ok";
+    case PK_ERR_ARG: return "invalid argument (null pointer, negative size or bad enum)";
+    case PK_ERR_SHAPE: return "shape not supported by the kernels";
+    case PK_ERR_ALIGN: return "pointer or leading dimension is not 16-byte aligned";
+    case PK_ERR_WORKSPACE: return "workspace too small";
+    case PK_ERR_UNSUPPORTED: return "dtype/option combination not supported";
+    default: return status > 0 ? "HIP runtime error (status is the hipError_t value)" : "unknown status";
+  }
+}
+
+int pk_gate_logits(const void* x, int x_dtype, const float* w_gate, const float* gate_bias,
+                   float* logits, int64_t T, int64_t H, int64_t E, pk_stream_t stream) {
+  if (T < 0 || H <= 0 || E <= 0 || !pk_dtype_ok(x_dtype)) return PK_ERR_ARG;
+  if (T == 0) return PK_OK;
+  if (!x || !w_gate || !logits) return PK_ERR_ARG;
+  if (T * E > 0x7fffffffll) return PK_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  if (gate_bias) {
+    const int64_t n = T * E;
+    hipLaunchKernelGGL(bias_fill_kernel, dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
+                       logits, gate_bias, T, (int)E);
+    PK_RETURN_IF_LAUNCH_FAILED();
+  }
+  pk_simt::Params p = {};
+  p.A = x; p.B = w_gate; p.C = logits;
+  p.ragged = pk_simt::RAGGED_NONE; p.G = 1; p.accumulate = gate_bias ? 1 : 0;
+  p.M = T; p.N = E; p.K = H;
+  p.sam = H; p.sak = 1; p.sbk = 1; p.sbn = H; p.scm = E; p.scn = 1;
+  return x_dtype == PK_BF16 ? pk_simt::launch<bf16_t, float, float>(p, s)
+                            : pk_simt::launch<float, float, float>(p, s);
+}
+
+int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const float* w_gate,
+                       float* d_x_f32, float* d_w_gate, float* d_gate_bias, int accumulate,
+                       int64_t T, int64_t H, int64_t E, pk_stream_t stream) {
+  if (T < 0 || H <= 0 || E <= 0 || !pk_dtype_ok(x_dtype)) return PK_ERR_ARG;
+  if (!d_logits && T > 0) return PK_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  if (d_x_f32 && T > 0) {
+    if (!w_gate) return PK_ERR_ARG;
+    pk_simt::Params p = {};
+    p.A = d_logits; p.B = w_gate; p.C = d_x_f32;
+    p.ragged = pk_simt::RAGGED_NONE; p.G = 1; p.accumulate = 0;
+    p.M = T; p.N = H; p.K = E;
+    p.sam = E; p.sak = 1; p.sbk = H; p.sbn = 1; p.scm = H; p.scn = 1;
+    int rc = pk_simt::launch<float, float, float>(p, s);
+    if (rc != PK_OK) return rc;
+  }
+  if (d_w_gate) {
+    if (!x && T > 0) return PK_ERR_ARG;
+    pk_simt::Params p = {};
+    p.A = d_logits; p.B = x; p.C = d_w_gate;
+    p.ragged = pk_simt::RAGGED_NONE; p.G = 1; p.accumulate = accumulate ? 1 : 0;
+    p.M = E; p.N = H; p.K = T;
+    p.sam = 1; p.sak = E; p.sbk = H; p.sbn = 1; p.scm = H; p.scn = 1;
+    int rc = x_dtype == PK_BF16 ? pk_simt::launch<float, bf16_t, float>(p, s)
+                                : pk_simt::launch<float, float, float>(p, s);
+    if (rc != PK_OK) return rc;
+  }
+  if (d_gate_bias) {
+    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)E), dim3(256), 0, s, d_logits, T, (int)E,
+                       d_gate_bias, accumulate ? 1 : 0);
+    PK_RETURN_IF_LAUNCH_FAILED();
+  }
+  return PK_OK;
+}
+
+#define PK_DISPATCH_EPL(E, LAUNCH)                 \
+  do {                                             \
+    if ((E) <= 64) { LAUNCH(1); }                  \
+    else if ((E) <= 128) { LAUNCH(2); }            \
+    else if ((E) <= 256) { LAUNCH(4); }            \
+    else if ((E) <= 512) { LAUNCH(8); }            \
+    else { LAUNCH(16); }                           \
+  } while (0)
+
+int pk_route_topk(const float* logits, int64_t T, int64_t E, int64_t K, int route_norm,
+                  float route_scale, float* top_scores, int32_t* top_idx, pk_stream_t stream) {
+  if (T < 0 || E <= 0 || K <= 0) return PK_ERR_ARG;
+  if (E > PK_MAX_EXPERTS || K > PK_MAX_TOPK || K > E) return PK_ERR_SHAPE;
+  if (T == 0) return PK_OK;
+  if (!logits || !top_scores || !top_idx) return PK_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)pk_ceil_div(T, kRouteThreads / 64)), block(kRouteThreads);
+#define PK_LAUNCH_TOPK(EPL)                                                                 \
+  hipLaunchKernelGGL((route_topk_kernel<EPL>), grid, block, 0, s, logits, (int)T, (int)E,   \
+                     (int)K, route_norm, route_scale, top_scores, top_idx)
+  PK_DISPATCH_EPL(E, PK_LAUNCH_TOPK);
+#undef PK_LAUNCH_TOPK
+  PK_RETURN_IF_LAUNCH_FAILED();
+  return PK_OK;
+}
+
+int pk_route_topk_bwd(const float* logits, const int32_t* top_idx, const float* d_top_scores,
+                      int64_t T, int64_t E, int64_t K, int route_norm, float route_scale,
+                      float* d_logits, pk_stream_t stream) {
+  if (T < 0 || E <= 0 || K <= 0) return PK_ERR_ARG;
+  if (E > PK_MAX_EXPERTS || K > PK_MAX_TOPK || K > E) return PK_ERR_SHAPE;
+  if (T == 0) return PK_OK;
+  if (!logits || !top_idx || !d_top_scores || !d_logits) return PK_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)pk_ceil_div(T, kRouteThreads / 64)), block(kRouteThreads);
+#define PK_LAUNCH_TOPK_BWD(EPL)                                                              \
+  hipLaunchKernelGGL((route_topk_bwd_kernel<EPL>), grid, block, 0, s, logits, top_idx,       \
+                     d_top_scores, (int)T, (int)E, (int)K, route_norm, route_scale, d_logits)
+  PK_DISPATCH_EPL(E, PK_LAUNCH_TOPK_BWD);
+#undef PK_LAUNCH_TOPK_BWD
+  PK_RETURN_IF_LAUNCH_FAILED();
+  return PK_OK;
+}
+
+int64_t pk_sort_workspace_bytes(int64_t A, int64_t E) {
+  if (A < 0 || E <= 0) return PK_ERR_ARG;
+  const int64_t nchunks = pk_ceil_div(A > 0 ? A : 1, kSortChunk);
+  return nchunks * E * (int64_t)sizeof(int32_t);
+}
+
+int pk_sort_by_expert(const int32_t* top_idx, int64_t A, int64_t E, int32_t* counts,
+                      int32_t* starts, int32_t* perm, int32_t* inv_perm, void* workspace,
+                      int64_t workspace_bytes, pk_stream_t stream) {
+  if (A < 0 || E <= 0) return PK_ERR_ARG;
+  if (E > PK_MAX_EXPERTS || A > 0x7fffffffll) return PK_ERR_SHAPE;
+  if (!starts || !workspace || (A > 0 && (!top_idx || !perm))) return PK_ERR_ARG;
+  if (workspace_bytes < pk_sort_workspace_bytes(A, E)) return PK_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  const int nchunks = (int)pk_ceil_div(A > 0 ? A : 1, kSortChunk);
+  int32_t* chunk_hist = reinterpret_cast<int32_t*>(workspace);
+  const size_t lds = (size_t)E * sizeof(int32_t);
+  hipLaunchKernelGGL(sort_hist_kernel, dim3(nchunks), dim3(64), lds, s, top_idx, (int)A, (int)E,
+                     chunk_hist);
+  PK_RETURN_IF_LAUNCH_FAILED();
+  hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(1024), 0, s, chunk_hist, nchunks, (int)E,
+                     counts, starts);
+  PK_RETURN_IF_LAUNCH_FAILED();
+  if (A > 0) {
+    hipLaunchKernelGGL(sort_scatter_kernel, dim3(nchunks), dim3(64), lds, s, top_idx, (int)A,
+                       (int)E, chunk_hist, perm, inv_perm);
+    PK_RETURN_IF_LAUNCH_FAILED();
+  }
+  return PK_OK;
+}
+
+int pk_counts_to_starts(const void* counts, int counts_is_i64, int64_t E, int32_t* starts,
+                        pk_stream_t stream) {
+  if (E <= 0 || !counts || !starts) return PK_ERR_ARG;
+  if (E > PK_MAX_EXPERTS) return PK_ERR_SHAPE;
+  hipLaunchKernelGGL(counts_to_starts_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, counts,
+                     counts_is_i64, (int)E, starts);
+  PK_RETURN_IF_LAUNCH_FAILED();
+  return PK_OK;
+}
+
+}  // extern "C"

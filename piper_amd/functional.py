@@ -1,0 +1,210 @@
+"""Autograd wiring of the expert region and registration of the reference's operator.
+
+Two ways in:
+
+* ``expert_region(...)``: the whole region (gate -> top-k -> sort -> grouped SwiGLU with the permute
+  fused into the operand load -> unpermute+combine) as ONE autograd node with a hand-written
+  backward.  This is what ``piper_amd.moe.AnnotatedMoE`` runs.
+* the piecewise operators the reference model code calls one by one
+  (examples/models/qwen3.py:237-283): ``router``, ``reorder``, ``permute``, ``bmm_experts``,
+  ``combine``.  ``bmm_experts`` is also registered as ``torch.ops.piper_artifact.bmm_experts`` with
+  the reference's schema (examples/models/qwen3_bmm_experts_patch.py:63-72), so reference model
+  code that looks the op up by name gets the HIP implementation.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+
+# --------------------------------------------------------------------------- piecewise operators
+
+
+class _RouterFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, w_gate, gate_bias, top_k, route_norm, route_scale):
+        logits = ops.gate_logits(x, w_gate, gate_bias)
+        top_scores, top_idx = ops.route_topk(logits, top_k, route_norm, route_scale)
+        ctx.save_for_backward(x, w_gate, logits, top_idx)
+        ctx.has_bias = gate_bias is not None
+        ctx.cfg = (route_norm, route_scale)
+        ctx.mark_non_differentiable(top_idx)
+        return top_scores, top_idx
+
+    @staticmethod
+    def backward(ctx, d_scores, _d_idx):
+        x, w_gate, logits, top_idx = ctx.saved_tensors
+        route_norm, route_scale = ctx.cfg
+        d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
+        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        d_w = torch.empty_like(w_gate) if need_dw else None
+        d_b = torch.empty(w_gate.shape[0], dtype=torch.float32, device=x.device) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        d_x32 = ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=need_dx, d_w_gate=d_w, d_gate_bias=d_b)
+        d_x = d_x32.to(x.dtype) if need_dx else None
+        return d_x, d_w, d_b, None, None, None
+
+
+def router(x, w_gate, gate_bias=None, *, top_k: int, route_norm: bool, route_scale: float = 1.0):
+    """(top_scores [T,K] f32, selected_experts_indices [T,K] i32, num_tokens_per_expert [E] i32).
+    The call `self.router(x, self.expert_bias)` of qwen3.py:237-241."""
+    top_scores, top_idx = _RouterFn.apply(x, w_gate, gate_bias, top_k, route_norm, route_scale)
+    # histogram without a host sync (torch.bincount reads the maximum back to size its output)
+    flat = top_idx.reshape(-1)
+    counts = torch.zeros(w_gate.shape[0], dtype=torch.int32, device=flat.device)
+    counts.index_add_(0, flat, torch.ones_like(flat))
+    return top_scores, top_idx, counts
+
+
+def reorder(top_scores: torch.Tensor, top_idx: torch.Tensor, num_experts: int):
+    """The reorderer of qwen3.py:243-247.  Returns (top_scores_experts_sorted [A],
+    token_indices_experts_sorted [A] i32, num_tokens_per_expert [E] i32)."""
+    counts, _starts, perm, _inv = ops.sort_by_expert(top_idx, num_experts)
+    scores_sorted = top_scores.reshape(-1)[perm.long()]
+    return scores_sorted, perm, counts
+
+
+class _PermuteFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, perm, top_k):
+        ctx.top_k = top_k
+        ctx.save_for_backward(perm)
+        return ops.permute_fwd(x, perm, top_k)
+
+    @staticmethod
+    def backward(ctx, d_routed):
+        (perm,) = ctx.saved_tensors
+        inv = torch.empty_like(perm)
+        inv[perm.long()] = torch.arange(perm.numel(), dtype=perm.dtype, device=perm.device)
+        return ops.permute_bwd(d_routed, inv, ctx.top_k), None, None
+
+
+def permute(x: torch.Tensor, token_indices_experts_sorted: torch.Tensor, top_k: int) -> torch.Tensor:
+    """routed_input = x[token_indices_experts_sorted // top_k]  (qwen3.py:250)."""
+    return _PermuteFn.apply(x, token_indices_experts_sorted, top_k)
+
+
+class _BmmExpertsFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, w1, w2, w3, x, num_tokens_per_expert):
+        starts = ops.counts_to_starts(num_tokens_per_expert)
+        y, g, u, h = ops.grouped_swiglu_fwd(x, w1, w2, w3, starts)
+        ctx.save_for_backward(w1, w2, w3, x, starts, g, u, h)
+        return y
+
+    @staticmethod
+    def backward(ctx, d_y):
+        w1, w2, w3, x, starts, g, u, h = ctx.saved_tensors
+        d_x, d_g, d_u = ops.grouped_swiglu_dgrad(d_y, w1, w2, w3, g, u, starts)
+        d_w1 = d_w2 = d_w3 = None
+        if any(ctx.needs_input_grad[:3]):
+            d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, w1.shape[0])
+        return d_w1, d_w2, d_w3, d_x, None
+
+
+def _bmm_experts_autograd(w1, w2, w3, x, num_tokens_per_expert):
+    if x.is_meta:
+        return torch.empty_like(x)
+    return _BmmExpertsFn.apply(w1, w2, w3, x, num_tokens_per_expert)
+
+
+def _bmm_experts_forward_only(w1, w2, w3, x, num_tokens_per_expert):
+    starts = ops.counts_to_starts(num_tokens_per_expert)
+    return ops.grouped_swiglu_fwd(x, w1, w2, w3, starts)[0]
+
+
+def _bmm_experts_meta(w1, w2, w3, x, num_tokens_per_expert):
+    return torch.empty_like(x)
+
+
+_LIBS = []
+
+
+def register_reference_op() -> bool:
+    """Define ``piper_artifact::bmm_experts`` (same schema as qwen3_bmm_experts_patch.py:63-65) on
+    the CUDA(=HIP)/Autograd/Meta keys.  If the op already exists (the reference patch was imported
+    first) only the CUDA and AutogradCUDA kernels are overridden.  Returns True when this call
+    registered something."""
+    if _LIBS:
+        return False
+    exists = hasattr(torch.ops, "piper_artifact") and hasattr(torch.ops.piper_artifact, "bmm_experts")
+    if not exists:
+        def_lib = torch.library.Library("piper_artifact", "DEF")
+        def_lib.define(
+            "bmm_experts(Tensor w1, Tensor w2, Tensor w3, Tensor x, Tensor num_tokens_per_expert) -> Tensor"
+        )
+        _LIBS.append(def_lib)
+    impl = torch.library.Library("piper_artifact", "IMPL")
+    impl.impl("bmm_experts", _bmm_experts_forward_only, "CUDA")
+    impl.impl("bmm_experts", _bmm_experts_autograd, "AutogradCUDA")
+    if not exists:
+        impl.impl("bmm_experts", _bmm_experts_meta, "Meta")
+    _LIBS.append(impl)
+    return True
+
+
+def bmm_experts(w1, w2, w3, x, num_tokens_per_expert):
+    """Same call as the reference's ``bmm_experts`` (qwen3_bmm_experts_patch.py:78-87)."""
+    register_reference_op()
+    return torch.ops.piper_artifact.bmm_experts(w1, w2, w3, x, num_tokens_per_expert)
+
+
+class _CombineFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, y_sorted, perm, top_scores):
+        inv = torch.empty_like(perm)
+        inv[perm.long()] = torch.arange(perm.numel(), dtype=perm.dtype, device=perm.device)
+        ctx.save_for_backward(y_sorted, perm, top_scores)
+        return ops.combine_fwd(y_sorted, inv, top_scores)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        y_sorted, perm, top_scores = ctx.saved_tensors
+        d_y, d_scores = ops.combine_bwd(d_out, y_sorted, perm, top_scores)
+        return d_y, None, d_scores
+
+
+def combine(gathered_output, token_indices_experts_sorted, top_scores):
+    """Unpermute scatter + fp32 weighted sum over k (qwen3.py:265-283), fused."""
+    return _CombineFn.apply(gathered_output, token_indices_experts_sorted, top_scores)
+
+
+# --------------------------------------------------------------------------- fused region
+
+
+class _ExpertRegionFn(torch.autograd.Function):
+    """x [T,H] -> out [T,H]; saves the routing tables and the SwiGLU pre-activations."""
+
+    @staticmethod
+    def forward(ctx, x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale):
+        E = w1.shape[0]
+        logits = ops.gate_logits(x, w_gate, gate_bias)
+        top_scores, top_idx = ops.route_topk(logits, top_k, route_norm, route_scale)
+        _counts, starts, perm, inv_perm = ops.sort_by_expert(top_idx, E)
+        y, g, u, h = ops.grouped_swiglu_fwd(x, w1, w2, w3, starts, row_map=perm, row_map_div=top_k)
+        out = ops.combine_fwd(y, inv_perm, top_scores)
+        ctx.save_for_backward(x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, h, y)
+        ctx.cfg = (top_k, route_norm, route_scale, gate_bias is not None)
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        (x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, h, y) = ctx.saved_tensors
+        top_k, route_norm, route_scale, has_bias = ctx.cfg
+        E = w1.shape[0]
+        need = ctx.needs_input_grad
+        d_y, d_scores = ops.combine_bwd(d_out, y, perm, top_scores)
+        d_xs, d_g, d_u = ops.grouped_swiglu_dgrad(d_y, w1, w2, w3, g, u, starts)
+        d_w1 = d_w2 = d_w3 = None
+        if need[3] or need[4] or need[5]:
+            d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k)
+        d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
+        d_wg = torch.empty_like(w_gate) if need[1] else None
+        d_b = torch.empty(E, dtype=torch.float32, device=x.device) if (has_bias and need[2]) else None
+        d_x32 = ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=need[0], d_w_gate=d_wg, d_gate_bias=d_b)
+        d_x = ops.permute_bwd(d_xs, inv_perm, top_k, addend_f32=d_x32) if need[0] else None
+        return d_x, d_wg, d_b, d_w1, d_w2, d_w3, None, None, None
+
+
+def expert_region(x, w_gate, gate_bias, w1, w2, w3, *, top_k: int, route_norm: bool, route_scale: float = 1.0):
+    """The whole MoE expert region of AnnotatedMoE.forward (qwen3.py:233-289) on x [T,H]."""
+    return _ExpertRegionFn.apply(x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale)
