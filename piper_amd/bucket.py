@@ -80,8 +80,7 @@ def flatten_params(bucket: BucketState, params: Sequence[torch.nn.Parameter], *,
     for p, off in zip(params, offsets):
         n = p.numel()
         p.data = flat_params[off:off + n].view(p.shape)
-        p.requires_grad_(True)
-        p.grad_dtype = grad_dtype
+        p.requires_grad_(True)  # gradients stay in the parameter dtype; the pack kernel widens them
         view_specs.append((p, off, n, tuple(p.shape)))
 
     shard_param = flat_params[0:padded]

@@ -1,0 +1,146 @@
+"""GPU parity of the grouped SwiGLU expert kernels (forward, input gradient, weight gradient)
+against the CPU oracle.  bf16 results are judged against the oracle evaluated in fp32 on the
+same bf16 inputs (tolerance 2e-2 of the output's maximum), fp32 results to 1e-5."""
+import pytest
+import torch
+
+from conftest import BF16_TOL, F32_TOL, rel_err
+from oracle import moe as O
+from piper_amd import functional as F_
+from piper_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _make(seed, counts, H, I, dtype):
+    g = torch.Generator().manual_seed(seed)
+    E = len(counts)
+    A = int(sum(counts))
+    x = torch.randn(A, H, generator=g).to(dtype)
+    w1 = (torch.randn(E, I, H, generator=g) * 0.05).to(dtype)
+    w3 = (torch.randn(E, I, H, generator=g) * 0.05).to(dtype)
+    w2 = (torch.randn(E, H, I, generator=g) * 0.05).to(dtype)
+    dy = torch.randn(A, H, generator=g).to(dtype)
+    return x, w1, w2, w3, dy, torch.tensor(counts, dtype=torch.long)
+
+
+def _oracle(x, w1, w2, w3, dy, counts):
+    """fp32 evaluation with autograd; also returns the SwiGLU intermediates' gradients."""
+    xr, w1r, w2r, w3r = (t.float().requires_grad_(True) for t in (x, w1, w2, w3))
+    y = O.grouped_swiglu(w1r, w2r, w3r, xr, counts)
+    dx, dw1, dw2, dw3 = torch.autograd.grad(y, (xr, w1r, w2r, w3r), dy.float())
+    return y.detach(), dx, dw1, dw2, dw3
+
+
+CASES = [
+    # (counts, H, I)   -- ragged, empty experts, single rows, more than one 128-row tile
+    ([128, 128, 128, 128], 256, 256),
+    ([0, 5, 300, 0, 129, 1, 127, 0], 256, 128),
+    ([37] * 16, 128, 384),
+    ([0, 0, 0, 700], 384, 256),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("counts,H,I", CASES)
+def test_grouped_swiglu_fwd_dgrad_wgrad(dev, dtype, counts, H, I):
+    print(f"[case] grouped_swiglu {dtype} counts={counts[:8]} H={H} I={I}", flush=True)
+    x, w1, w2, w3, dy, cnt = _make(3, counts, H, I, dtype)
+    y_ref, dx_ref, dw1_ref, dw2_ref, dw3_ref = _oracle(x, w1, w2, w3, dy, cnt)
+    tol = BF16_TOL if dtype == torch.bfloat16 else F32_TOL
+    E = len(counts)
+    X, W1, W2, W3, DY = (t.to(dev) for t in (x, w1, w2, w3, dy))
+    starts = ops.counts_to_starts(cnt.to(dev))
+    y, g, u, h = ops.grouped_swiglu_fwd(X, W1, W2, W3, starts)
+    assert y.dtype == dtype and rel_err(y, y_ref) <= tol
+    # saved pre-activations are what they claim to be
+    if sum(counts) > 0:
+        e0 = next(e for e, c in enumerate(counts) if c > 0)
+        s0 = int(sum(counts[:e0]))
+        g_ref = x[s0:s0 + counts[e0]].float() @ w1[e0].float().t()
+        assert rel_err(g[s0:s0 + counts[e0]], g_ref) <= tol
+    dx, dg, du = ops.grouped_swiglu_dgrad(DY, W1, W2, W3, g, u, starts)
+    assert rel_err(dx, dx_ref) <= tol
+    dw1, dw2, dw3 = ops.grouped_swiglu_wgrad(DY, h, dg, du, X, starts, E)
+    assert rel_err(dw1, dw1_ref) <= tol and rel_err(dw2, dw2_ref) <= tol and rel_err(dw3, dw3_ref) <= tol
+    for e, c in enumerate(counts):
+        if c == 0:  # an expert without rows gets exact zeros, not garbage
+            assert float(dw1[e].abs().max()) == 0.0 and float(dw2[e].abs().max()) == 0.0 and float(dw3[e].abs().max()) == 0.0
+    # accumulate=True adds a second microbatch on top
+    ops.grouped_swiglu_wgrad(DY, h, dg, du, X, starts, E, d_w1=dw1, d_w2=dw2, d_w3=dw3, accumulate=True)
+    assert rel_err(dw2, 2 * dw2_ref) <= tol and rel_err(dw1, 2 * dw1_ref) <= tol
+
+
+def test_mfma_path_agrees_with_fma_path(dev):
+    """bf16 shapes outside the MFMA tiling (H or I not a multiple of 128) run on the FMA kernel."""
+    print("[case] bf16 fallback shapes", flush=True)
+    counts = [10, 0, 70, 3]
+    x, w1, w2, w3, dy, cnt = _make(4, counts, 192, 64, torch.bfloat16)
+    y_ref, dx_ref, dw1_ref, dw2_ref, dw3_ref = _oracle(x, w1, w2, w3, dy, cnt)
+    X, W1, W2, W3, DY = (t.to(dev) for t in (x, w1, w2, w3, dy))
+    starts = ops.counts_to_starts(cnt.to(dev))
+    y, g, u, h = ops.grouped_swiglu_fwd(X, W1, W2, W3, starts)
+    dx, dg, du = ops.grouped_swiglu_dgrad(DY, W1, W2, W3, g, u, starts)
+    dw1, dw2, dw3 = ops.grouped_swiglu_wgrad(DY, h, dg, du, X, starts, 4)
+    for a, b in ((y, y_ref), (dx, dx_ref), (dw1, dw1_ref), (dw2, dw2_ref), (dw3, dw3_ref)):
+        assert rel_err(a, b) <= BF16_TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_fused_permute_operand_load(dev, dtype):
+    """row_map = perm, div = K: reading x[perm[p] // K] inside the GEMM equals permute then GEMM."""
+    print(f"[case] fused permute {dtype}", flush=True)
+    T, H, I, E, K = 300, 256, 128, 8, 2
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(T, E, generator=g)
+    logits[:, 3] = -50.0
+    _, idx = O.route_topk(logits, K, True)
+    counts, starts_ref, perm, inv = O.sort_by_expert(idx, E)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    _, w1, w2, w3, _, _ = _make(6, [1] * E, H, I, dtype)
+    X, W1, W2, W3 = (t.to(dev) for t in (x, w1, w2, w3))
+    starts = starts_ref.int().to(dev)
+    P = perm.int().to(dev)
+    routed = ops.permute_fwd(X, P, K)
+    y_a, g_a, u_a, h_a = ops.grouped_swiglu_fwd(routed, W1, W2, W3, starts)
+    y_b, g_b, u_b, h_b = ops.grouped_swiglu_fwd(X, W1, W2, W3, starts, row_map=P, row_map_div=K)
+    assert torch.equal(y_a, y_b) and torch.equal(g_a, g_b) and torch.equal(h_a, h_b)
+    dy = torch.randn(T * K, H, generator=g).to(dtype).to(dev)
+    dx, dg, du = ops.grouped_swiglu_dgrad(dy, W1, W2, W3, g_a, u_a, starts)
+    wa = ops.grouped_swiglu_wgrad(dy, h_a, dg, du, routed, starts, E)
+    wb = ops.grouped_swiglu_wgrad(dy, h_a, dg, du, X, starts, E, row_map=P, row_map_div=K)
+    for a, b in zip(wa, wb):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("counts_dtype", [torch.int64, torch.int32])
+def test_reference_operator_bmm_experts(dev, counts_dtype):
+    """torch.ops.piper_artifact.bmm_experts(w1, w2, w3, x, num_tokens_per_expert) with autograd:
+    the reference's operator boundary (qwen3_bmm_experts_patch.py:63-87)."""
+    print("[case] piper_artifact::bmm_experts", flush=True)
+    counts = [60, 0, 200, 4]
+    x, w1, w2, w3, dy, cnt = _make(8, counts, 256, 128, torch.bfloat16)
+    y_ref, dx_ref, dw1_ref, dw2_ref, dw3_ref = _oracle(x, w1, w2, w3, dy, cnt)
+    F_.register_reference_op()
+    X, W1, W2, W3 = (t.to(dev).requires_grad_(True) for t in (x, w1, w2, w3))
+    y = torch.ops.piper_artifact.bmm_experts(W1, W2, W3, X, cnt.to(counts_dtype).to(dev))
+    assert y.shape == x.shape and rel_err(y, y_ref) <= BF16_TOL
+    y.backward(dy.to(dev))
+    assert rel_err(X.grad, dx_ref) <= BF16_TOL
+    assert rel_err(W1.grad, dw1_ref) <= BF16_TOL and rel_err(W2.grad, dw2_ref) <= BF16_TOL and rel_err(W3.grad, dw3_ref) <= BF16_TOL
+    with torch.no_grad():
+        y2 = torch.ops.piper_artifact.bmm_experts(W1, W2, W3, X, cnt.to(counts_dtype).to(dev))
+    assert torch.equal(y2, y.detach())
+    meta = torch.ops.piper_artifact.bmm_experts(*(t.detach().to("meta") for t in (W1, W2, W3, X)), cnt.to("meta"))
+    assert meta.shape == x.shape and meta.is_meta
+
+
+def test_argument_errors(dev):
+    z = torch.zeros(4, 8, device=dev, dtype=torch.bfloat16)
+    w = torch.zeros(2, 16, 8, device=dev, dtype=torch.bfloat16)
+    w2 = torch.zeros(2, 8, 16, device=dev, dtype=torch.bfloat16)
+    starts = torch.tensor([0, 2, 4], dtype=torch.int32, device=dev)
+    with pytest.raises(ValueError):
+        ops.grouped_swiglu_fwd(z, w, w, w, starts)             # w2 has the wrong shape
+    with pytest.raises(ValueError):
+        ops.grouped_swiglu_fwd(z.float(), w, w2, w, starts)    # dtype mismatch

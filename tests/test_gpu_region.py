@@ -1,0 +1,213 @@
+"""Whole expert region (router -> sort -> grouped SwiGLU -> combine, forward and backward) on the
+GPU against the CPU oracle, at config 1 exactly and at a reduced config 3; config 3 / 4 at full
+size are checked through size-independent properties."""
+import pytest
+import torch
+
+from conftest import ADAMW_TOL, BF16_TOL, F32_TOL, rel_err
+from oracle import bucket as OB
+from oracle import moe as O
+from piper_amd import functional as F_
+from piper_amd import ops
+from piper_amd.bucket import BucketState, ParamStorage, StageStore, flatten_params
+from piper_amd.configs import ADAMW, CFG1, CFG3, CFG4, ExpertRegionConfig, make_expert_region_inputs
+from piper_amd.moe import AnnotatedMoE, MoEArgs
+from piper_amd.optim import FusedAdamW
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_fwd_bwd(inp, cfg, compute_dtype=None):
+    names = ("x", "w_gate", "w1", "w2", "w3")
+    leaves = {k: inp[k].clone().float().requires_grad_(True) if compute_dtype else inp[k].clone().requires_grad_(True)
+              for k in names}
+    bias = inp["gate_bias"].clone().requires_grad_(True) if inp["gate_bias"] is not None else None
+    out, aux = O.moe_forward(leaves["x"], leaves["w_gate"], bias, leaves["w1"], leaves["w2"], leaves["w3"],
+                             cfg.top_k, cfg.route_norm, cfg.route_scale, compute_dtype=compute_dtype)
+    targets = [leaves[k] for k in names] + ([bias] if bias is not None else [])
+    grads = torch.autograd.grad(out, targets, inp["d_out"].to(out.dtype))
+    g = dict(zip(names, grads))
+    if bias is not None:
+        g["gate_bias"] = grads[-1]
+    return out.detach(), aux, g
+
+
+def _gpu_fwd_bwd(inp, cfg, dev, fused=True):
+    t = {k: (v.to(dev).requires_grad_(True) if v is not None and k != "d_out" else v) for k, v in inp.items()}
+    if fused:
+        out = F_.expert_region(t["x"], t["w_gate"], t["gate_bias"], t["w1"], t["w2"], t["w3"],
+                               top_k=cfg.top_k, route_norm=cfg.route_norm, route_scale=cfg.route_scale)
+    else:
+        E = cfg.num_experts
+        ts, ti, cnt = F_.router(t["x"], t["w_gate"], t["gate_bias"], top_k=cfg.top_k, route_norm=cfg.route_norm,
+                                route_scale=cfg.route_scale)
+        _ss, perm, cnt2 = F_.reorder(ts, ti, E)
+        assert torch.equal(cnt, cnt2)
+        routed = F_.permute(t["x"], perm, cfg.top_k)
+        y = F_.bmm_experts(t["w1"], t["w2"], t["w3"], routed, cnt2)
+        out = F_.combine(y, perm, ts)
+    out.backward(inp["d_out"].to(dev))
+    g = {k: t[k].grad for k in ("x", "w_gate", "w1", "w2", "w3")}
+    if t["gate_bias"] is not None:
+        g["gate_bias"] = t["gate_bias"].grad
+    return out.detach(), g
+
+
+def test_config1_exact_four_microbatches_then_bucket_adamw(dev):
+    """Config 1 as specified: fp32, 4 microbatches x 256 tokens, fwd+bwd, all grads flattened into
+    one bucket, one AdamW step."""
+    cfg = CFG1
+    names = ("w_gate", "w1", "w3", "w2")
+    acc_ref = None
+    inp0 = make_expert_region_inputs(cfg, microbatch=0)
+    params = {k: torch.nn.Parameter(inp0[k].clone().to(dev)) for k in names}
+    for mb in range(cfg.microbatches):
+        print(f"[case] cfg1 microbatch {mb}", flush=True)
+        inp = make_expert_region_inputs(cfg, microbatch=mb)
+        out_ref, aux, g_ref = _oracle_fwd_bwd(inp, cfg)
+        x = inp["x"].to(dev).requires_grad_(True)
+        out = F_.expert_region(x, params["w_gate"], None, params["w1"], params["w2"], params["w3"],
+                               top_k=cfg.top_k, route_norm=cfg.route_norm)
+        # routing tables bit-exact (checked through the piecewise operators on the same input)
+        logits = ops.gate_logits(x.detach(), params["w_gate"].detach())
+        _, idx = ops.route_topk(logits, cfg.top_k, cfg.route_norm)
+        assert torch.equal(idx.cpu().long(), aux["top_idx"])
+        counts, starts, perm, inv = ops.sort_by_expert(idx, cfg.num_experts)
+        assert torch.equal(perm.cpu().long(), aux["perm"]) and torch.equal(counts.cpu().long(), aux["counts"])
+        assert rel_err(out, out_ref) <= F32_TOL
+        out.backward(inp["d_out"].to(dev))
+        assert rel_err(x.grad, g_ref["x"]) <= F32_TOL
+        acc_ref = {k: g_ref[k] if acc_ref is None else acc_ref[k] + g_ref[k] for k in names}
+        for k in names:
+            assert rel_err(params[k].grad, acc_ref[k]) <= F32_TOL, k
+    # flatten every gradient into one bucket and take one AdamW step
+    store = StageStore()
+    store.buckets[0] = BucketState()
+    store.zero_managed_ubids.add(0)
+    plist = [params[k] for k in names]
+    grads = [p.grad for p in plist]
+    flatten_params(store.buckets[0], plist, optim_class=lambda ps: FusedAdamW(ps, **ADAMW))
+    for p, gr in zip(plist, grads):
+        p.grad = gr
+    ps = ParamStorage(store)
+    ps.accumulate_zero_param_grads_to_flat(0, None)
+    ps.step_zero_shard_optimizers(None, {})
+    numels = [inp0[k].numel() for k in names]
+    assert sum(numels) == 3_147_776
+    offs, total = OB.plan_offsets(numels, 4, 256)
+    assert [s[1] for s in store.buckets[0].param_view_specs] == offs
+    master = OB.flatten([inp0[k] for k in names], offs, total, torch.float32)
+    flat_g = OB.pack(torch.zeros(total), [acc_ref[k] for k in names], offs)
+    z = torch.zeros(total)
+    ref_master, _, _ = OB.adamw_step_torch(master, flat_g, z, z, 1, ADAMW["lr"], ADAMW["betas"], ADAMW["eps"], ADAMW["weight_decay"])
+    got = store.buckets[0].flat_params.cpu()
+    # Step 1 of Adam moves each weight by ~lr*sign(g): where the oracle's gradient is ~0 the sign is
+    # noise, so compare where |g| is resolved and bound the rest by the step size.
+    resolved = flat_g.abs() > 1e-6
+    assert (got - ref_master)[resolved].abs().max().item() <= 2e-5
+    assert (got - ref_master).abs().max().item() <= 2.1 * ADAMW["lr"]
+    # with the GPU's own gradient bucket the optimizer arithmetic itself is exact to 1e-6
+    ref2, _, _ = OB.adamw_step_torch(master, store.buckets[0].flat_grads.cpu(), z, z, 1, ADAMW["lr"], ADAMW["betas"], ADAMW["eps"], ADAMW["weight_decay"])
+    assert (got - ref2).abs().max().item() <= ADAMW_TOL
+
+
+SMALL_BF16 = ExpertRegionConfig("small-bf16", tokens=1024, hidden=256, num_experts=16, top_k=4, inter=128,
+                                dtype=torch.bfloat16, zipf_s=1.2, zipf_alpha=1.5)
+REDUCED_CFG3 = ExpertRegionConfig("cfg3-reduced", tokens=512, hidden=2048, num_experts=128, top_k=8, inter=768,
+                                  dtype=torch.bfloat16)
+
+
+@pytest.mark.parametrize("cfg", [SMALL_BF16, REDUCED_CFG3], ids=lambda c: c.name)
+@pytest.mark.parametrize("fused", [True, False])
+def test_bf16_region_against_fp32_oracle(dev, cfg, fused):
+    print(f"[case] region {cfg.name} fused={fused}", flush=True)
+    inp = make_expert_region_inputs(cfg)
+    out_ref, aux, g_ref = _oracle_fwd_bwd(inp, cfg, compute_dtype=torch.float32)
+    out, g = _gpu_fwd_bwd(inp, cfg, dev, fused=fused)
+    assert out.dtype == torch.bfloat16
+    assert rel_err(out, out_ref) <= BF16_TOL
+    for k in g_ref:
+        assert rel_err(g[k], g_ref[k]) <= BF16_TOL, k
+    if cfg.zipf_s is not None:
+        assert int((aux["counts"] == 0).sum()) > 0, "this case is meant to contain empty experts"
+
+
+def test_fused_and_piecewise_paths_agree(dev):
+    inp = make_expert_region_inputs(SMALL_BF16)
+    o1, g1 = _gpu_fwd_bwd(inp, SMALL_BF16, dev, fused=True)
+    o2, g2 = _gpu_fwd_bwd(inp, SMALL_BF16, dev, fused=False)
+    assert torch.equal(o1, o2)
+    for k in g1:
+        assert rel_err(g1[k], g2[k]) <= 1e-2, k
+
+
+def test_module_mirrors_reference_layer(dev):
+    """AnnotatedMoE with the reference's parameter names runs both data flows."""
+    args = MoEArgs(num_experts=8, top_k=2, route_norm=True)
+    torch.manual_seed(0)
+    moe = AnnotatedMoE(args, dim=256, hidden_dim=128, dtype=torch.bfloat16).to(dev)
+    moe.init_weights()
+    assert {n for n, _ in moe.named_parameters()} == {"router.gate.weight", "experts.w1", "experts.w2", "experts.w3"}
+    x = torch.randn(2, 64, 256, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    y1 = moe(x)
+    moe.fused = False
+    y2 = moe(x)
+    assert y1.shape == x.shape and torch.equal(y1, y2)
+    y1.float().sum().backward()
+    assert moe.experts.w1.grad is not None and moe.router.gate.weight.grad.dtype == torch.float32
+
+
+@pytest.mark.parametrize("cfg", [CFG3, CFG4], ids=lambda c: c.name)
+def test_full_size_properties(dev, cfg):
+    """Full-size configs: routing invariants, spot-checked experts against a GPU fp32 matmul of the
+    same rows, linearity of the backward in the upstream gradient, exact zero grads for row-less experts."""
+    print(f"[case] full size {cfg.name}", flush=True)
+    inp = make_expert_region_inputs(cfg)
+    E, K, T = cfg.num_experts, cfg.top_k, cfg.tokens
+    d = {k: (v.to(dev) if v is not None else None) for k, v in inp.items()}
+    logits = ops.gate_logits(d["x"], d["w_gate"], d["gate_bias"])
+    scores, idx = ops.route_topk(logits, K, True)
+    counts, starts, perm, inv = ops.sort_by_expert(idx, E)
+    # routing invariants
+    assert int(counts.sum()) == T * K and int(starts[-1]) == T * K
+    assert torch.equal(torch.sort(perm).values, torch.arange(T * K, device=dev, dtype=torch.int32))
+    e_sorted = idx.reshape(-1)[perm.long()]
+    assert bool((e_sorted[1:] >= e_sorted[:-1]).all())
+    same = e_sorted[1:] == e_sorted[:-1]
+    assert bool((perm[1:][same] > perm[:-1][same]).all())
+    assert torch.allclose(scores.sum(1), torch.ones(T, device=dev), atol=1e-5)
+    # CPU oracle on the GPU's logits: bit-exact tables
+    s_ref, i_ref = O.route_topk(logits.cpu(), K, True)
+    assert torch.equal(idx.cpu().long(), i_ref)
+    c_ref, st_ref, p_ref, _ = O.sort_by_expert(i_ref, E)
+    assert torch.equal(perm.cpu().long(), p_ref) and torch.equal(counts.cpu().long(), c_ref)
+    if cfg.zipf_s is not None:
+        top8 = torch.sort(c_ref, descending=True).values[:8].sum().item() / (T * K)
+        assert 0.35 <= top8 <= 0.45, f"Zipf skew: top-8 experts hold {top8:.3f} of the assignments"
+    # experts forward / backward, spot-check three experts against fp32 matmuls of the same rows
+    y, g, u, h = ops.grouped_swiglu_fwd(d["x"], d["w1"], d["w2"], d["w3"], starts, row_map=perm, row_map_div=K)
+    dy = torch.randn(T * K, cfg.hidden, device=dev, dtype=cfg.dtype, generator=torch.Generator(device=dev).manual_seed(1))
+    dx, dg, du = ops.grouped_swiglu_dgrad(dy, d["w1"], d["w2"], d["w3"], g, u, starts)
+    dw1, dw2, dw3 = ops.grouped_swiglu_wgrad(dy, h, dg, du, d["x"], starts, E, row_map=perm, row_map_div=K)
+    order = torch.argsort(c_ref)
+    for e in (int(order[0]), int(order[E // 2]), int(order[-1])):
+        s0, s1 = int(st_ref[e]), int(st_ref[e + 1])
+        if s1 == s0:
+            assert float(dw1[e].abs().max()) == 0.0
+            continue
+        rows = (perm[s0:s1].long() // K)
+        xe = d["x"][rows].float().requires_grad_(True)
+        w1e, w2e, w3e = (d[k][e].float().requires_grad_(True) for k in ("w1", "w2", "w3"))
+        ye = (torch.nn.functional.silu(xe @ w1e.t()) * (xe @ w3e.t())) @ w2e.t()
+        gx, g1, g2, g3 = torch.autograd.grad(ye, (xe, w1e, w2e, w3e), dy[s0:s1].float())
+        assert rel_err(y[s0:s1], ye) <= BF16_TOL
+        assert rel_err(dx[s0:s1], gx) <= BF16_TOL
+        assert rel_err(dw1[e], g1) <= BF16_TOL and rel_err(dw2[e], g2) <= BF16_TOL and rel_err(dw3[e], g3) <= BF16_TOL
+    # whole region: linear in the upstream gradient (scale by 2 -> every gradient doubles)
+    out1, g1_ = _gpu_fwd_bwd(inp, cfg, dev)
+    inp2 = dict(inp)
+    inp2["d_out"] = inp["d_out"] * 2
+    out2, g2_ = _gpu_fwd_bwd(inp2, cfg, dev)
+    assert torch.equal(out1, out2)
+    for k in g1_:
+        assert rel_err(g2_[k], 2 * g1_[k].float()) <= 1e-2, k

@@ -1,0 +1,166 @@
+"""GPU parity of the routing kernels against the CPU oracle: indices, permutation and offsets are
+compared bit-exactly, scores and gradients to the fp32 tolerance."""
+import pytest
+import torch
+
+from conftest import F32_TOL, rel_err
+from oracle import moe as O
+from piper_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _note(msg):
+    print(f"[case] {msg}", flush=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,H,E,bias", [(256, 256, 8, False), (1000, 2048, 128, True), (3, 40, 5, True)])
+def test_gate_logits(dev, dtype, T, H, E, bias):
+    _note(f"gate_logits {dtype} T={T} H={H} E={E} bias={bias}")
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    w = torch.randn(E, H, generator=g) * 0.02
+    b = torch.randn(E, generator=g) if bias else None
+    got = ops.gate_logits(x.to(dev), w.to(dev), None if b is None else b.to(dev))
+    ref = O.gate_logits(x, w, b)
+    assert got.dtype == torch.float32
+    assert rel_err(got, ref) <= F32_TOL
+
+
+def _check_topk(dev, logits, K, route_norm, scale=1.0):
+    s_ref, i_ref = O.route_topk(logits, K, route_norm, scale)
+    s, i = ops.route_topk(logits.to(dev), K, route_norm, scale)
+    assert i.dtype == torch.int32
+    assert torch.equal(i.cpu().long(), i_ref), "routing indices must be bit-exact"
+    assert rel_err(s, s_ref) <= F32_TOL
+    return s, i
+
+
+@pytest.mark.parametrize("T,E,K", [(4096, 128, 8), (1027, 8, 2), (64, 64, 64), (33, 200, 6), (10, 1024, 64), (5, 3, 1), (7, 65, 65 - 1)])
+@pytest.mark.parametrize("route_norm", [True, False])
+def test_route_topk_random(dev, T, E, K, route_norm):
+    _note(f"route_topk random T={T} E={E} K={K} norm={route_norm}")
+    g = torch.Generator().manual_seed(T + E + K)
+    _check_topk(dev, torch.randn(T, E, generator=g) * 0.9, min(K, 64), route_norm, 1.0 if route_norm else 2.5)
+
+
+def test_route_topk_ties_to_lower_index(dev):
+    _note("route_topk ties")
+    g = torch.Generator().manual_seed(5)
+    T, E, K = 2048, 128, 8
+    # heavy quantisation: many exact ties in every row
+    logits = torch.round(torch.randn(T, E, generator=g) * 2.0) / 2.0
+    logits[0] = 0.0                       # all equal -> experts 0..7
+    logits[1] = 0.0
+    logits[1, 5] = -0.0                   # signed zero is still a tie
+    logits[2] = torch.arange(E).float()   # strictly increasing -> highest indices, descending
+    logits[3, :] = -3.0
+    logits[3, 100:] = 7.0                 # 28 equal maxima -> 100..107
+    s, i = _check_topk(dev, logits, K, True)
+    i = i.cpu()
+    assert i[0].tolist() == list(range(8)) and i[1].tolist() == list(range(8))
+    assert i[2].tolist() == list(range(127, 119, -1))
+    assert i[3].tolist() == list(range(100, 108))
+
+
+def test_route_topk_argument_errors(dev):
+    logits = torch.zeros(4, 8, device=dev)
+    with pytest.raises(RuntimeError, match="shape"):
+        ops.route_topk(logits, 9, True)          # K > E
+    with pytest.raises(RuntimeError, match="shape"):
+        ops.route_topk(torch.zeros(2, 2000, device=dev), 2, True)   # E > 1024
+    s, i = ops.route_topk(torch.zeros(0, 8, device=dev), 2, True)    # empty input is fine
+    assert s.shape == (0, 2)
+
+
+@pytest.mark.parametrize("T,E,K,empty", [(4096, 128, 8, False), (16384, 128, 8, True), (37, 8, 2, True), (1, 5, 3, False), (700, 1024, 4, True), (64, 8, 8, False)])
+def test_sort_by_expert_bit_exact(dev, T, E, K, empty):
+    _note(f"sort T={T} E={E} K={K} empty={empty}")
+    g = torch.Generator().manual_seed(T * 7 + E)
+    logits = torch.randn(T, E, generator=g)
+    if empty:
+        logits[:, E // 2] = -100.0      # an expert that receives nothing
+        logits[:, 0] += 3.0             # and a very popular one
+    _, idx = O.route_topk(logits, K, True)
+    c_ref, s_ref, p_ref, inv_ref = O.sort_by_expert(idx, E)
+    counts, starts, perm, inv = ops.sort_by_expert(idx.int().to(dev), E)
+    assert torch.equal(counts.cpu().long(), c_ref)
+    assert torch.equal(starts.cpu().long(), s_ref)
+    assert torch.equal(perm.cpu().long(), p_ref), "permutation order must be bit-exact"
+    assert torch.equal(inv.cpu().long(), inv_ref)
+    if empty:
+        assert counts[E // 2].item() == 0
+    st = ops.counts_to_starts(counts)
+    assert torch.equal(st.cpu(), starts.cpu())
+    st64 = ops.counts_to_starts(counts.long())
+    assert torch.equal(st64.cpu(), starts.cpu())
+
+
+def test_sort_with_repeated_expert_in_a_row(dev):
+    # the sort itself does not require distinct experts per token
+    _note("sort duplicates")
+    g = torch.Generator().manual_seed(9)
+    idx = torch.randint(0, 16, (999, 4), generator=g)
+    ref = O.sort_by_expert(idx, 16)
+    got = ops.sort_by_expert(idx.int().to(dev), 16)
+    for a, b in zip(got, ref):
+        assert torch.equal(a.cpu().long(), b)
+
+
+@pytest.mark.parametrize("route_norm", [True, False])
+@pytest.mark.parametrize("T,E,K", [(512, 128, 8), (100, 8, 2), (9, 300, 5)])
+def test_route_topk_backward(dev, T, E, K, route_norm):
+    _note(f"route_topk_bwd T={T} E={E} K={K} norm={route_norm}")
+    g = torch.Generator().manual_seed(11)
+    logits = (torch.randn(T, E, generator=g) * 0.9).requires_grad_(True)
+    d_scores = torch.randn(T, K, generator=g)
+    s_ref, i_ref = O.route_topk(logits, K, route_norm, 1.5)
+    (d_ref,) = torch.autograd.grad(s_ref, logits, d_scores)
+    got = ops.route_topk_bwd(logits.detach().to(dev), i_ref.int().to(dev), d_scores.to(dev), route_norm, 1.5)
+    assert rel_err(got, d_ref) <= F32_TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gate_logits_backward(dev, dtype):
+    _note(f"gate_logits_bwd {dtype}")
+    g = torch.Generator().manual_seed(12)
+    T, H, E = 777, 256, 24
+    x = torch.randn(T, H, generator=g).to(dtype)
+    w = (torch.randn(E, H, generator=g) * 0.02)
+    d_logits = torch.randn(T, E, generator=g)
+    xr = x.float().requires_grad_(True)
+    wr = w.clone().requires_grad_(True)
+    br = torch.zeros(E, requires_grad=True)
+    ref = O.gate_logits(xr, wr, br)
+    dx_ref, dw_ref, db_ref = torch.autograd.grad(ref, (xr, wr, br), d_logits)
+    dw = torch.zeros(E, H, device=dev)
+    db = torch.zeros(E, device=dev)
+    dx = ops.gate_logits_bwd(d_logits.to(dev), x.to(dev), w.to(dev), True, dw, db, accumulate=False)
+    assert rel_err(dx, dx_ref) <= F32_TOL and rel_err(dw, dw_ref) <= F32_TOL and rel_err(db, db_ref) <= F32_TOL
+    # accumulate adds on top
+    ops.gate_logits_bwd(d_logits.to(dev), x.to(dev), w.to(dev), False, dw, db, accumulate=True)
+    assert rel_err(dw, 2 * dw_ref) <= F32_TOL and rel_err(db, 2 * db_ref) <= F32_TOL
+
+
+def test_end_to_end_routing_from_activations(dev):
+    """x, W -> indices.  The GPU gate sums in a different order than the CPU, so logits differ in
+    the last bits; every index that differs from the oracle must sit on a near-tie (margin below
+    1e-4), and given the GPU's own logits the selection is bit-exact."""
+    _note("routing end to end (cfg3 shape)")
+    from piper_amd.configs import CFG3, make_expert_region_inputs
+    inp = make_expert_region_inputs(CFG3)
+    x, w = inp["x"], inp["w_gate"]
+    logits_gpu = ops.gate_logits(x.to(dev), w.to(dev)).cpu()
+    logits_ref = O.gate_logits(x, w)
+    assert rel_err(logits_gpu, logits_ref) <= F32_TOL
+    _, i_gpu = ops.route_topk(logits_gpu.to(dev), 8, True)
+    _, i_from_gpu_logits = O.route_topk(logits_gpu, 8, True)
+    assert torch.equal(i_gpu.cpu().long(), i_from_gpu_logits)
+    _, i_ref = O.route_topk(logits_ref, 8, True)
+    diff_rows = (i_gpu.cpu().long() != i_ref).any(dim=1).nonzero().flatten()
+    srt = torch.sort(logits_ref, dim=1, descending=True).values
+    gaps = (srt[:, :8] - srt[:, 1:9])          # margins that decide order and membership
+    for r in diff_rows.tolist():
+        assert gaps[r].min().item() < 1e-4, f"row {r} differs without a near-tie"
+    assert len(diff_rows) <= 8
