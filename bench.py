@@ -1,0 +1,247 @@
+#!/usr/bin/env python3
+"""Headline benchmark: expert-region forward+backward tokens/s on the Qwen3-30B-A3B-shaped
+configuration (one microbatch of 4096 tokens per step), with the roofline of its dominant kernel,
+the ZeRO bucket path (pack + fused AdamW) in GB/s, and the CPU oracle timed on the host cores.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg4] [--no-cpu-baseline]
+
+Prints ONE JSON line.  Inputs are synthetic (seed 0), generated on the host and resident in HBM
+before the timed region starts.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", choices=["cfg3", "cfg4"], default="cfg3")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-bucket", action="store_true")
+    return ap.parse_args()
+
+
+def kernel_flops(cfg) -> dict:
+    """Algorithmic flops of ONE launch of each GEMM kernel: 2*A*H*I per GEMM."""
+    one = 2.0 * cfg.routed_rows * cfg.hidden * cfg.inter
+    return {
+        "swiglu_gate_up": 2 * one,   # gate and up projections in one launch
+        "swiglu_down": one,
+        "swiglu_dgrad_dh": one,
+        "swiglu_dgrad_dx": 2 * one,  # d_g.w1 + d_u.w3
+        "swiglu_wgrad": 3 * one,     # d_w1, d_w2, d_w3 in one launch
+    }
+
+
+def bench_region(cfg, steps: int, warmup: int):
+    import torch
+
+    from piper_amd import _lib, functional as F_
+    from piper_amd.configs import make_expert_region_inputs
+
+    dev = torch.device("cuda:0")
+    inp = make_expert_region_inputs(cfg)
+    x = inp["x"].to(dev).requires_grad_(True)
+    w_gate = inp["w_gate"].to(dev).requires_grad_(True)
+    bias = inp["gate_bias"].to(dev).requires_grad_(True) if inp["gate_bias"] is not None else None
+    w1, w2, w3 = (inp[k].to(dev).requires_grad_(True) for k in ("w1", "w2", "w3"))
+    d_out = inp["d_out"].to(dev)
+    leaves = [t for t in (x, w_gate, bias, w1, w2, w3) if t is not None]
+
+    def step():
+        for t in leaves:          # clear_param_grads: first microbatch of an iteration
+            t.grad = None
+        out = F_.expert_region(x, w_gate, bias, w1, w2, w3, top_k=cfg.top_k, route_norm=cfg.route_norm,
+                               route_scale=cfg.route_scale)
+        out.backward(d_out)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.timing_enable(True)
+    _lib.timing_collect()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    records = _lib.timing_collect()
+    _lib.timing_enable(False)
+
+    per_kernel: dict = {}
+    for name, ms in records:
+        tot, n = per_kernel.get(name, (0.0, 0))
+        per_kernel[name] = (tot + ms, n + 1)
+    summary = {k: {"launches_per_step": n / steps, "avg_ms": tot / n, "ms_per_step": tot / steps}
+               for k, (tot, n) in per_kernel.items()}
+    return elapsed, summary
+
+
+def bench_bucket(steps: int, warmup: int):
+    """Config 2: 96 bf16 gradient tensors -> fp32 bucket (one pack launch), fused AdamW over the
+    whole bucket writing the fp32 master and the bf16 parameter bucket the views alias."""
+    import torch
+
+    from piper_amd import _lib, ops
+    from piper_amd.configs import ADAMW, bucket_manifest_cfg2
+
+    dev = torch.device("cuda:0")
+    manifest = bucket_manifest_cfg2()
+    shapes = [s for _, s in manifest]
+    numels = [math.prod(s) for s in shapes]
+    offs, total = ops.bucket_plan(numels, 2, 256)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    grads = [(torch.randn(s, device=dev, generator=gen) * 1e-3).bfloat16() for s in shapes]
+    flat_g = torch.zeros(total, device=dev)
+    master = torch.randn(total, device=dev, generator=gen) * 0.02
+    m = torch.zeros_like(master)
+    v = torch.zeros_like(master)
+    shadow = master.bfloat16()
+    state = {"step": 0}
+
+    def step():
+        state["step"] += 1
+        ops.bucket_pack(grads, offs, flat_g, accumulate=False)
+        ops.adamw_fused(master, m, v, flat_g, step=state["step"], lr=ADAMW["lr"], beta1=ADAMW["betas"][0],
+                        beta2=ADAMW["betas"][1], eps=ADAMW["eps"], weight_decay=ADAMW["weight_decay"], shadow=shadow)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.timing_enable(True)
+    _lib.timing_collect()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    records = _lib.timing_collect()
+    _lib.timing_enable(False)
+    n_elems = sum(numels)
+    pack_ms = [ms for k, ms in records if k == "bucket_pack"]
+    adam_ms = [ms for k, ms in records if k == "adamw"]
+    pack_avg, adam_avg = sum(pack_ms) / len(pack_ms), sum(adam_ms) / len(adam_ms)
+    pack_bytes = 6.0 * n_elems            # read bf16 grad, write fp32 bucket
+    adam_bytes = 30.0 * total             # read g,p,m,v (16) + write p,m,v (12) + bf16 parameter (2)
+    agg_gbs = (pack_bytes + adam_bytes) * steps / elapsed / 1e9
+    return {
+        "metric": "bucket pack + fused AdamW HBM GB/s",
+        "value": agg_gbs, "unit": "GB/s", "ms_per_step": elapsed / steps * 1e3,
+        "config": {"workload": "cfg2: 96 tensors of two Qwen3-30B-A3B layers, bf16 grads / fp32 master",
+                   "tensors": len(shapes), "elements": n_elems, "bucket_elements": total},
+        "bytes_per_element": {"pack": 6, "adamw": 30},
+        "pack": {"avg_ms": pack_avg, "GB/s": pack_bytes / pack_avg / 1e6, "frac": pack_bytes / pack_avg / 1e6 / HBM_PEAK_GBS},
+        "adamw": {"avg_ms": adam_avg, "GB/s": adam_bytes / adam_avg / 1e6, "frac": adam_bytes / adam_avg / 1e6 / HBM_PEAK_GBS},
+        "roofline": {"bound": "hbm", "achieved": agg_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": agg_gbs / HBM_PEAK_GBS, "traffic": None},
+    }
+
+
+def cpu_baseline(cfg):
+    """The CPU oracle (un-padded per-expert loop, fp32) on a bounded sample of the same workload:
+    the first tokens of the microbatch with the full set of experts."""
+    import torch
+
+    from oracle import moe as O
+    from piper_amd.configs import make_expert_region_inputs
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    sample_tokens = min(cfg.tokens, 512)
+    inp = make_expert_region_inputs(cfg)
+    names = ("x", "w_gate", "w1", "w2", "w3")
+
+    def one():
+        leaves = {k: (inp[k][:sample_tokens] if k == "x" else inp[k]).float().requires_grad_(True) for k in names}
+        bias = inp["gate_bias"]
+        out, _ = O.moe_forward(leaves["x"], leaves["w_gate"], bias, leaves["w1"], leaves["w2"], leaves["w3"], cfg.top_k,
+                               cfg.route_norm, cfg.route_scale, compute_dtype=torch.float32)
+        torch.autograd.grad(out, list(leaves.values()), inp["d_out"][:sample_tokens].float())
+
+    one()  # warm-up
+    times = []
+    for _ in range(2):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[0]
+    return {"value": sample_tokens / t, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"first {sample_tokens} of {cfg.tokens} tokens, all {cfg.num_experts} experts, fp32 per-expert loop, "
+                      f"fwd+bwd, best of 2 after 1 warm-up ({t:.2f} s per pass)"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no collectives, run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from piper_amd import _lib
+    from piper_amd.configs import CFG3, CFG4
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    _lib.load()
+    cfg = CFG3 if args.workload == "cfg3" else CFG4
+    elapsed, kernels = bench_region(cfg, args.steps, args.warmup)
+    ms_per_step = elapsed / args.steps * 1e3
+    tokens_per_s = cfg.tokens * args.steps / elapsed
+    gemm_flops_step = cfg.gemm_flops_per_token * cfg.tokens
+    mfma_frac_region = gemm_flops_step / (ms_per_step * 1e-3) / (MFMA_BF16_PEAK_TFLOPS * 1e12)
+
+    flops = kernel_flops(cfg)
+    gemm_kernels = {k: v for k, v in kernels.items() if k in flops}
+    dominant = max(gemm_kernels, key=lambda k: gemm_kernels[k]["ms_per_step"])
+    dom = gemm_kernels[dominant]
+    achieved = flops[dominant] / (dom["avg_ms"] * 1e-3) / 1e12
+    result = {
+        "metric": "expert-region fwd+bwd tokens/s",
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: T={cfg.tokens} H={cfg.hidden} E={cfg.num_experts} top{cfg.top_k} "
+                               f"I={cfg.inter}, bf16 experts, fp32 router, fwd+bwd incl. router and all expert weight grads",
+                   "tokens_per_step": cfg.tokens},
+        "mfma_frac_of_peak_region": mfma_frac_region,
+        "gemm_tflops_region": gemm_flops_step / (ms_per_step * 1e-3) / 1e12,
+        "roofline": {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "flops_per_launch": flops[dominant], "avg_launch_ms": dom["avg_ms"]},
+        "kernels_ms_per_step": {k: round(v["ms_per_step"], 4) for k, v in sorted(kernels.items(), key=lambda kv: -kv[1]["ms_per_step"])},
+        "gemm_kernels_tflops": {k: round(flops[k] / (v["avg_ms"] * 1e-3) / 1e12, 1) for k, v in gemm_kernels.items()},
+    }
+    if not args.no_bucket:
+        result["bucket"] = bench_bucket(max(5, args.steps), max(2, args.warmup))
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(cfg)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -214,6 +214,15 @@ PK_API int pk_adamw_fused(float* master, float* exp_avg, float* exp_avg_sq, floa
                    float weight_decay, int64_t step, float grad_scale, int zero_grad,
                    pk_stream_t stream);
 
+/* ------------------------------------------------------------- kernel timing
+ * Measurement aid with no counterpart in the reference: when enabled, every kernel launch of
+ * the library is bracketed by two hipEventRecord calls on its stream.  pk_timing_collect
+ * waits for the recorded events, writes up to max_records (kernel id, milliseconds) pairs in
+ * launch order, forgets them and returns how many launches were recorded. */
+PK_API int pk_timing_enable(int on);
+PK_API int64_t pk_timing_collect(int32_t* ids, float* ms, int64_t max_records);
+PK_API const char* pk_timing_kernel_name(int id);
+
 #ifdef __cplusplus
 }
 #endif

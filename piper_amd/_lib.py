@@ -49,6 +49,9 @@ SIGNATURES = {
     "pk_bucket_zero": (_c_int, [_p, _c_i64, _p]),
     "pk_adamw_fused": (_c_int, [_p, _p, _p, _p, _p, _c_int, _c_i64, _c_f32, _c_f32, _c_f32, _c_f32,
                                 _c_f32, _c_i64, _c_f32, _c_int, _p]),
+    "pk_timing_enable": (_c_int, [_c_int]),
+    "pk_timing_collect": (_c_i64, [_p, _p, _c_i64]),
+    "pk_timing_kernel_name": (C.c_char_p, [_c_int]),
 }
 
 _lib = None
@@ -86,6 +89,20 @@ def call(name: str, *args):
     if rc != 0:
         raise RuntimeError(f"{name} failed with status {rc}: {status_string(rc)}")
     return rc
+
+
+def timing_enable(on: bool) -> None:
+    """Switch per-kernel HIP-event timing inside the library on or off."""
+    load().pk_timing_enable(int(bool(on)))
+
+
+def timing_collect(max_records: int = 1 << 16) -> list[tuple[str, float]]:
+    """Wait for and return the (kernel name, milliseconds) records since the last collect."""
+    lib = load()
+    ids = (C.c_int32 * max_records)()
+    ms = (C.c_float * max_records)()
+    n = min(int(lib.pk_timing_collect(ids, ms, max_records)), max_records)
+    return [(lib.pk_timing_kernel_name(ids[i]).decode(), float(ms[i])) for i in range(n)]
 
 
 def dtype_code(dtype: torch.dtype) -> int:

@@ -15,7 +15,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libpiper_amd.so"
-SOURCES = ["bucket.hip", "route.hip", "permute.hip", "grouped_gemm.hip"]
+SOURCES = ["bucket.hip", "route.hip", "permute.hip", "grouped_gemm.hip", "timing.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -59,7 +59,7 @@ def build_library(verbose: bool = False) -> Path:
     if verbose:
         for c in cmds:
             print(" ".join(c))
-    with ThreadPoolExecutor(max_workers=min(4, len(cmds))) as pool:
+    with ThreadPoolExecutor(max_workers=min(5, len(cmds))) as pool:
         list(pool.map(_run, cmds))
     tmp = LIB_PATH.with_suffix(".so.tmp")
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *objs])

@@ -110,7 +110,7 @@ __global__ __launch_bounds__(kPackThreads) void pack_kernel(const PackArgs args,
 
 template <typename TS, typename TD, bool ACC, bool TO_FLAT>
 int launch_pack(const PackArgs& a, int nblocks, void* flat, hipStream_t s) {
-  hipLaunchKernelGGL((pack_kernel<TS, TD, ACC, TO_FLAT>), dim3(nblocks), dim3(kPackThreads), 0, s,
+  PK_LAUNCH_NOCHECK(TO_FLAT ? pk_timing::K_BUCKET_PACK : pk_timing::K_BUCKET_UNPACK, s, (pack_kernel<TS, TD, ACC, TO_FLAT>), dim3(nblocks), dim3(kPackThreads), 0, s,
                      a, flat);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
@@ -305,7 +305,7 @@ int pk_bucket_zero(float* flat, int64_t n, pk_stream_t stream) {
   if (n < 0 || (n > 0 && !flat)) return PK_ERR_ARG;
   if (n == 0) return PK_OK;
   if (!pk_aligned16(flat)) return PK_ERR_ALIGN;
-  hipLaunchKernelGGL(zero_kernel, dim3(stream_grid(n >> 2)), dim3(kStreamThreads), 0,
+  PK_LAUNCH_NOCHECK(pk_timing::K_BUCKET_ZERO, (hipStream_t)stream, zero_kernel, dim3(stream_grid(n >> 2)), dim3(kStreamThreads), 0,
                      (hipStream_t)stream, flat, n);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
@@ -337,7 +337,7 @@ int pk_adamw_fused(float* master, float* exp_avg, float* exp_avg_sq, float* grad
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(stream_grid(n >> 2)), block(kStreamThreads);
 #define PK_ADAM_LAUNCH(TSH, SH, ZE)                                                          \
-  hipLaunchKernelGGL((adamw_kernel<TSH, SH, ZE>), grid, block, 0, s, master, exp_avg,        \
+  PK_LAUNCH_NOCHECK(pk_timing::K_ADAMW, s, (adamw_kernel<TSH, SH, ZE>), grid, block, 0, s, master, exp_avg,        \
                      exp_avg_sq, grad, reinterpret_cast<TSH*>(shadow), n, a)
   if (!shadow) {
     if (zero_grad) PK_ADAM_LAUNCH(float, false, true); else PK_ADAM_LAUNCH(float, false, false);

@@ -386,10 +386,10 @@ __global__ __launch_bounds__(THREADS) void wgrad_kernel(const WgradParams p) {
 inline int round_up_xcd(int64_t n) { return (int)(pk_ceil_div(n, NXCD) * NXCD); }
 
 template <bool B_KCONTIG, int EPI>
-int launch_ragged_m(RaggedMParams p, int64_t A_rows, hipStream_t s) {
+int launch_ragged_m(RaggedMParams p, int64_t A_rows, int kernel_id, hipStream_t s) {
   const int64_t max_units = (pk_ceil_div(A_rows, BM) + p.E) * p.n_tiles;
   if (max_units > 0x7ffffff0ll) return PK_ERR_SHAPE;
-  hipLaunchKernelGGL((ragged_m_kernel<B_KCONTIG, EPI>), dim3(round_up_xcd(max_units)),
+  PK_LAUNCH_NOCHECK(kernel_id, s, (ragged_m_kernel<B_KCONTIG, EPI>), dim3(round_up_xcd(max_units)),
                      dim3(THREADS), 0, s, p);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
@@ -475,7 +475,7 @@ int fwd_simt(const void* x, const int32_t* row_map, int64_t div, const void* w1,
   rc = simt_ragged_m<T>(x, H, row_map, div, w3, 1, H, I * H, u, I, starts, A, I, H, E, 0, s);
   if (rc) return rc;
   const int64_t n = A * I;
-  hipLaunchKernelGGL((swiglu_fwd_kernel<T>), dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
+  PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_ELEMENTWISE, s, (swiglu_fwd_kernel<T>), dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
                      (const T*)g, (const T*)u, (T*)h, n);
   PK_RETURN_IF_LAUNCH_FAILED();
   return simt_ragged_m<T>(h, I, nullptr, 1, w2, 1, I, H * I, y, H, starts, A, H, I, E, 0, s);
@@ -489,7 +489,7 @@ int dgrad_simt(const void* dy, const void* w1, const void* w2, const void* w3, c
   int rc = simt_ragged_m<T>(dy, H, nullptr, 1, w2, I, 1, H * I, du, I, starts, A, I, H, E, 0, s);
   if (rc) return rc;
   const int64_t n = A * I;
-  hipLaunchKernelGGL((swiglu_bwd_kernel<T>), dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
+  PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_ELEMENTWISE, s, (swiglu_bwd_kernel<T>), dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
                      (const T*)du, (const T*)g, (const T*)u, (T*)dg, (T*)du, n);
   PK_RETURN_IF_LAUNCH_FAILED();
   // d_x = d_g . w1[e] + d_u . w3[e]   (w[e] is [I, H]: B(k=i, n=h) = w[i*H + h])
@@ -539,7 +539,7 @@ int pk_grouped_swiglu_fwd(const void* x_rows, const int32_t* row_map, int64_t ro
   p.starts = starts; p.E = (int32_t)E; p.Kseg = (int32_t)H; p.nseg = 1;
   p.n_tiles = (int32_t)(I / 64);
   p.O0 = (bf16_t*)g; p.O1 = (bf16_t*)u; p.O2 = (bf16_t*)h; p.ldc = I;
-  rc = mf::launch_ragged_m<true, mf::EPI_SWIGLU>(p, A, s);
+  rc = mf::launch_ragged_m<true, mf::EPI_SWIGLU>(p, A, pk_timing::K_SWIGLU_GATE_UP, s);
   if (rc) return rc;
 
   mf::RaggedMParams q = {};
@@ -548,7 +548,7 @@ int pk_grouped_swiglu_fwd(const void* x_rows, const int32_t* row_map, int64_t ro
   q.starts = starts; q.E = (int32_t)E; q.Kseg = (int32_t)I; q.nseg = 1;
   q.n_tiles = (int32_t)(H / mf::BN);
   q.O0 = (bf16_t*)y; q.ldc = H;
-  return mf::launch_ragged_m<true, mf::EPI_PLAIN>(q, A, s);
+  return mf::launch_ragged_m<true, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DOWN, s);
 }
 
 int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, const void* w3,
@@ -574,7 +574,7 @@ int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, con
   p.n_tiles = (int32_t)(I / mf::BN);
   p.Gin = (const bf16_t*)g; p.Uin = (const bf16_t*)u;
   p.O0 = (bf16_t*)d_g; p.O1 = (bf16_t*)d_u; p.ldc = I;
-  rc = mf::launch_ragged_m<false, mf::EPI_SWIGLU_BWD>(p, A, s);
+  rc = mf::launch_ragged_m<false, mf::EPI_SWIGLU_BWD>(p, A, pk_timing::K_SWIGLU_DGRAD_DH, s);
   if (rc) return rc;
 
   // d_x = [d_g | d_u] . [w1[e] ; w3[e]]
@@ -584,7 +584,7 @@ int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, con
   q.starts = starts; q.E = (int32_t)E; q.Kseg = (int32_t)I; q.nseg = 2;
   q.n_tiles = (int32_t)(H / mf::BN);
   q.O0 = (bf16_t*)d_x_sorted; q.ldc = H;
-  return mf::launch_ragged_m<false, mf::EPI_PLAIN>(q, A, s);
+  return mf::launch_ragged_m<false, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DGRAD_DX, s);
 }
 
 int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, const void* d_u,
@@ -632,7 +632,7 @@ int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, con
   p.tiles_per_expert = (int32_t)((H / mf::BM) * (I / mf::BN));
   const int64_t blocks = (int64_t)p.tiles_per_expert * E;
   if (blocks > 0x7ffffff0ll) return PK_ERR_SHAPE;
-  hipLaunchKernelGGL(mf::wgrad_kernel, dim3(mf::round_up_xcd(blocks), n), dim3(mf::THREADS), 0, s, p);
+  PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_WGRAD, s, mf::wgrad_kernel, dim3(mf::round_up_xcd(blocks), n), dim3(mf::THREADS), 0, s, p);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
 }

@@ -135,11 +135,11 @@ int pk_permute_fwd(const void* x, int dtype, const int32_t* perm, void* routed, 
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)A);
   if (dtype == PK_BF16) {
-    if (vec) hipLaunchKernelGGL((permute_fwd_kernel<bf16_t, true>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)x, perm, (bf16_t*)routed, H, (int)K);
-    else hipLaunchKernelGGL((permute_fwd_kernel<bf16_t, false>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)x, perm, (bf16_t*)routed, H, (int)K);
+    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_PERMUTE_FWD, s, (permute_fwd_kernel<bf16_t, true>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)x, perm, (bf16_t*)routed, H, (int)K);
+    else PK_LAUNCH_NOCHECK(pk_timing::K_PERMUTE_FWD, s, (permute_fwd_kernel<bf16_t, false>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)x, perm, (bf16_t*)routed, H, (int)K);
   } else {
-    if (vec) hipLaunchKernelGGL((permute_fwd_kernel<float, true>), grid, dim3(kRowThreads), 0, s, (const float*)x, perm, (float*)routed, H, (int)K);
-    else hipLaunchKernelGGL((permute_fwd_kernel<float, false>), grid, dim3(kRowThreads), 0, s, (const float*)x, perm, (float*)routed, H, (int)K);
+    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_PERMUTE_FWD, s, (permute_fwd_kernel<float, true>), grid, dim3(kRowThreads), 0, s, (const float*)x, perm, (float*)routed, H, (int)K);
+    else PK_LAUNCH_NOCHECK(pk_timing::K_PERMUTE_FWD, s, (permute_fwd_kernel<float, false>), grid, dim3(kRowThreads), 0, s, (const float*)x, perm, (float*)routed, H, (int)K);
   }
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
@@ -156,11 +156,11 @@ static int gather_reduce(const void* rows, int dtype, const int32_t* inv_perm, c
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)T);
   if (dtype == PK_BF16) {
-    if (vec) hipLaunchKernelGGL((gather_reduce_kernel<bf16_t, true>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)rows, inv_perm, weights, addend, (bf16_t*)out, H, (int)K);
-    else hipLaunchKernelGGL((gather_reduce_kernel<bf16_t, false>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)rows, inv_perm, weights, addend, (bf16_t*)out, H, (int)K);
+    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<bf16_t, true>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)rows, inv_perm, weights, addend, (bf16_t*)out, H, (int)K);
+    else PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<bf16_t, false>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)rows, inv_perm, weights, addend, (bf16_t*)out, H, (int)K);
   } else {
-    if (vec) hipLaunchKernelGGL((gather_reduce_kernel<float, true>), grid, dim3(kRowThreads), 0, s, (const float*)rows, inv_perm, weights, addend, (float*)out, H, (int)K);
-    else hipLaunchKernelGGL((gather_reduce_kernel<float, false>), grid, dim3(kRowThreads), 0, s, (const float*)rows, inv_perm, weights, addend, (float*)out, H, (int)K);
+    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<float, true>), grid, dim3(kRowThreads), 0, s, (const float*)rows, inv_perm, weights, addend, (float*)out, H, (int)K);
+    else PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<float, false>), grid, dim3(kRowThreads), 0, s, (const float*)rows, inv_perm, weights, addend, (float*)out, H, (int)K);
   }
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
@@ -190,11 +190,11 @@ int pk_combine_bwd(const void* d_out, const void* y_sorted, int dtype, const int
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)A);
   if (dtype == PK_BF16) {
-    if (vec) hipLaunchKernelGGL((combine_bwd_kernel<bf16_t, true>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)d_out, (const bf16_t*)y_sorted, perm, top_scores, (bf16_t*)d_y_sorted, d_top_scores, H, (int)K);
-    else hipLaunchKernelGGL((combine_bwd_kernel<bf16_t, false>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)d_out, (const bf16_t*)y_sorted, perm, top_scores, (bf16_t*)d_y_sorted, d_top_scores, H, (int)K);
+    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_COMBINE_BWD, s, (combine_bwd_kernel<bf16_t, true>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)d_out, (const bf16_t*)y_sorted, perm, top_scores, (bf16_t*)d_y_sorted, d_top_scores, H, (int)K);
+    else PK_LAUNCH_NOCHECK(pk_timing::K_COMBINE_BWD, s, (combine_bwd_kernel<bf16_t, false>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)d_out, (const bf16_t*)y_sorted, perm, top_scores, (bf16_t*)d_y_sorted, d_top_scores, H, (int)K);
   } else {
-    if (vec) hipLaunchKernelGGL((combine_bwd_kernel<float, true>), grid, dim3(kRowThreads), 0, s, (const float*)d_out, (const float*)y_sorted, perm, top_scores, (float*)d_y_sorted, d_top_scores, H, (int)K);
-    else hipLaunchKernelGGL((combine_bwd_kernel<float, false>), grid, dim3(kRowThreads), 0, s, (const float*)d_out, (const float*)y_sorted, perm, top_scores, (float*)d_y_sorted, d_top_scores, H, (int)K);
+    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_COMBINE_BWD, s, (combine_bwd_kernel<float, true>), grid, dim3(kRowThreads), 0, s, (const float*)d_out, (const float*)y_sorted, perm, top_scores, (float*)d_y_sorted, d_top_scores, H, (int)K);
+    else PK_LAUNCH_NOCHECK(pk_timing::K_COMBINE_BWD, s, (combine_bwd_kernel<float, false>), grid, dim3(kRowThreads), 0, s, (const float*)d_out, (const float*)y_sorted, perm, top_scores, (float*)d_y_sorted, d_top_scores, H, (int)K);
   }
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;

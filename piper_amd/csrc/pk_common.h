@@ -25,6 +25,34 @@ static inline int64_t pk_ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b
 static inline size_t pk_dtype_size(int dtype) { return dtype == PK_BF16 ? 2 : 4; }
 static inline bool pk_dtype_ok(int dtype) { return dtype == PK_F32 || dtype == PK_BF16; }
 
+// ---------------------------------------------------------------- optional kernel timing
+namespace pk_timing {
+enum KernelId {
+  K_GATE_LOGITS = 0, K_ROUTE_TOPK, K_ROUTE_TOPK_BWD, K_GATE_LOGITS_BWD, K_SORT_HIST, K_SORT_SCAN,
+  K_SORT_SCATTER, K_COUNTS_TO_STARTS, K_PERMUTE_FWD, K_GATHER_REDUCE, K_COMBINE_BWD,
+  K_SWIGLU_GATE_UP, K_SWIGLU_DOWN, K_SWIGLU_DGRAD_DH, K_SWIGLU_DGRAD_DX, K_SWIGLU_WGRAD,
+  K_SIMT_GEMM, K_SWIGLU_ELEMENTWISE, K_BUCKET_PACK, K_BUCKET_UNPACK, K_BUCKET_ZERO, K_ADAMW,
+  K_MISC, K_COUNT
+};
+// Brackets one kernel launch with two event records on `s` when timing is enabled
+// (pk_timing_enable); otherwise does nothing.
+class Scope {
+ public:
+  Scope(int id, hipStream_t s);
+  ~Scope();
+ private:
+  hipStream_t stream_;
+  int slot_;
+};
+}  // namespace pk_timing
+
+// Launch a kernel under a timing scope (the caller checks hipGetLastError afterwards).
+#define PK_LAUNCH_NOCHECK(id, stream, ...)          \
+  do {                                              \
+    pk_timing::Scope pk_scope_((id), (stream));     \
+    hipLaunchKernelGGL(__VA_ARGS__);                \
+  } while (0)
+
 // ---------------------------------------------------------------- device helpers
 template <typename T>
 __device__ __forceinline__ float pk_to_float(T v);

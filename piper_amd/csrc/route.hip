@@ -306,7 +306,7 @@ int pk_gate_logits(const void* x, int x_dtype, const float* w_gate, const float*
   hipStream_t s = (hipStream_t)stream;
   if (gate_bias) {
     const int64_t n = T * E;
-    hipLaunchKernelGGL(bias_fill_kernel, dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
+    PK_LAUNCH_NOCHECK(pk_timing::K_MISC, s, bias_fill_kernel, dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
                        logits, gate_bias, T, (int)E);
     PK_RETURN_IF_LAUNCH_FAILED();
   }
@@ -347,7 +347,7 @@ int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const 
     if (rc != PK_OK) return rc;
   }
   if (d_gate_bias) {
-    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)E), dim3(256), 0, s, d_logits, T, (int)E,
+    PK_LAUNCH_NOCHECK(pk_timing::K_MISC, s, colsum_kernel, dim3((unsigned)E), dim3(256), 0, s, d_logits, T, (int)E,
                        d_gate_bias, accumulate ? 1 : 0);
     PK_RETURN_IF_LAUNCH_FAILED();
   }
@@ -372,7 +372,7 @@ int pk_route_topk(const float* logits, int64_t T, int64_t E, int64_t K, int rout
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)pk_ceil_div(T, kRouteThreads / 64)), block(kRouteThreads);
 #define PK_LAUNCH_TOPK(EPL)                                                                 \
-  hipLaunchKernelGGL((route_topk_kernel<EPL>), grid, block, 0, s, logits, (int)T, (int)E,   \
+  PK_LAUNCH_NOCHECK(pk_timing::K_ROUTE_TOPK, s, (route_topk_kernel<EPL>), grid, block, 0, s, logits, (int)T, (int)E,   \
                      (int)K, route_norm, route_scale, top_scores, top_idx)
   PK_DISPATCH_EPL(E, PK_LAUNCH_TOPK);
 #undef PK_LAUNCH_TOPK
@@ -390,7 +390,7 @@ int pk_route_topk_bwd(const float* logits, const int32_t* top_idx, const float* 
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)pk_ceil_div(T, kRouteThreads / 64)), block(kRouteThreads);
 #define PK_LAUNCH_TOPK_BWD(EPL)                                                              \
-  hipLaunchKernelGGL((route_topk_bwd_kernel<EPL>), grid, block, 0, s, logits, top_idx,       \
+  PK_LAUNCH_NOCHECK(pk_timing::K_ROUTE_TOPK_BWD, s, (route_topk_bwd_kernel<EPL>), grid, block, 0, s, logits, top_idx,       \
                      d_top_scores, (int)T, (int)E, (int)K, route_norm, route_scale, d_logits)
   PK_DISPATCH_EPL(E, PK_LAUNCH_TOPK_BWD);
 #undef PK_LAUNCH_TOPK_BWD
@@ -415,14 +415,14 @@ int pk_sort_by_expert(const int32_t* top_idx, int64_t A, int64_t E, int32_t* cou
   const int nchunks = (int)pk_ceil_div(A > 0 ? A : 1, kSortChunk);
   int32_t* chunk_hist = reinterpret_cast<int32_t*>(workspace);
   const size_t lds = (size_t)E * sizeof(int32_t);
-  hipLaunchKernelGGL(sort_hist_kernel, dim3(nchunks), dim3(64), lds, s, top_idx, (int)A, (int)E,
+  PK_LAUNCH_NOCHECK(pk_timing::K_SORT_HIST, s, sort_hist_kernel, dim3(nchunks), dim3(64), lds, s, top_idx, (int)A, (int)E,
                      chunk_hist);
   PK_RETURN_IF_LAUNCH_FAILED();
-  hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(1024), 0, s, chunk_hist, nchunks, (int)E,
+  PK_LAUNCH_NOCHECK(pk_timing::K_SORT_SCAN, s, sort_scan_kernel, dim3(1), dim3(1024), 0, s, chunk_hist, nchunks, (int)E,
                      counts, starts);
   PK_RETURN_IF_LAUNCH_FAILED();
   if (A > 0) {
-    hipLaunchKernelGGL(sort_scatter_kernel, dim3(nchunks), dim3(64), lds, s, top_idx, (int)A,
+    PK_LAUNCH_NOCHECK(pk_timing::K_SORT_SCATTER, s, sort_scatter_kernel, dim3(nchunks), dim3(64), lds, s, top_idx, (int)A,
                        (int)E, chunk_hist, perm, inv_perm);
     PK_RETURN_IF_LAUNCH_FAILED();
   }
@@ -433,7 +433,7 @@ int pk_counts_to_starts(const void* counts, int counts_is_i64, int64_t E, int32_
                         pk_stream_t stream) {
   if (E <= 0 || !counts || !starts) return PK_ERR_ARG;
   if (E > PK_MAX_EXPERTS) return PK_ERR_SHAPE;
-  hipLaunchKernelGGL(counts_to_starts_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, counts,
+  PK_LAUNCH_NOCHECK(pk_timing::K_COUNTS_TO_STARTS, (hipStream_t)stream, counts_to_starts_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, counts,
                      counts_is_i64, (int)E, starts);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;

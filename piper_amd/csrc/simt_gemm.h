@@ -153,7 +153,7 @@ inline int launch(Params p, hipStream_t s) {
   }
   if (grid.x == 0 || grid.y == 0) return PK_OK;
   if (grid.y > 65535u || grid.z > 65535u) return PK_ERR_SHAPE;
-  hipLaunchKernelGGL((gemm_kernel<TA, TB, TC>), grid, dim3(THREADS), 0, s, p);
+  PK_LAUNCH_NOCHECK(pk_timing::K_SIMT_GEMM, s, (gemm_kernel<TA, TB, TC>), grid, dim3(THREADS), 0, s, p);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
 }
