@@ -52,10 +52,14 @@ PK_API const char* pk_status_string(int status);
 /* ------------------------------------------------------------------ routing */
 
 /* logits[T,E] (f32) = x[T,H] (x_dtype) . w_gate[E,H]^T (f32) + gate_bias[E] (f32, may be NULL),
- * fp32 accumulation.  Replaces the gate Linear inside `self.router(x, expert_bias)`
+ * fp32 products and accumulation.  The hidden dimension is split over workgroups into
+ * `workspace` (pk_gate_workspace_bytes) and summed in a fixed order; without a workspace it
+ * runs unsplit.  Replaces the gate Linear inside `self.router(x, expert_bias)`
  * (examples/models/qwen3.py:237-241; MoEArgs.gate_bias at :45). */
+PK_API int64_t pk_gate_workspace_bytes(int64_t T, int64_t H, int64_t E);
 PK_API int pk_gate_logits(const void* x, int x_dtype, const float* w_gate, const float* gate_bias,
-                   float* logits, int64_t T, int64_t H, int64_t E, pk_stream_t stream);
+                   float* logits, int64_t T, int64_t H, int64_t E, void* workspace,
+                   int64_t workspace_bytes, pk_stream_t stream);
 
 /* Softmax over experts in fp32, top-K selection, optional renormalisation of the K
  * selected scores (route_norm) and scaling (route_scale).
@@ -77,10 +81,14 @@ PK_API int pk_route_topk_bwd(const float* logits, const int32_t* top_idx, const 
  *   d_x_f32[T,H]   (f32)  = d_logits . w_gate                (written, not accumulated)
  *   d_w_gate[E,H]  (f32) += or = d_logits^T . x              (accumulate != 0 adds)
  *   d_gate_bias[E] (f32) += or = column sums of d_logits     (may be NULL)
- * d_x_f32 or d_w_gate may be NULL to skip that product. */
+ * d_x_f32 or d_w_gate may be NULL to skip that product.  The token reduction of d_w_gate is
+ * split over workgroups into `workspace` (pk_gate_bwd_workspace_bytes) and summed in a fixed
+ * order; without a workspace it runs unsplit (slower, same result up to fp32 rounding). */
+PK_API int64_t pk_gate_bwd_workspace_bytes(int64_t T, int64_t H, int64_t E);
 PK_API int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const float* w_gate,
                        float* d_x_f32, float* d_w_gate, float* d_gate_bias, int accumulate,
-                       int64_t T, int64_t H, int64_t E, pk_stream_t stream);
+                       int64_t T, int64_t H, int64_t E, void* workspace, int64_t workspace_bytes,
+                       pk_stream_t stream);
 
 /* Stable counting sort of the A = T*K flat slots (slot = t*K + k) by expert id.
  *   counts[E]   i32  tokens per expert                          (histogram)

@@ -26,10 +26,12 @@ _p = C.c_void_p
 SIGNATURES = {
     "pk_version": (_c_int, []),
     "pk_status_string": (C.c_char_p, [_c_int]),
-    "pk_gate_logits": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_gate_workspace_bytes": (_c_i64, [_c_i64, _c_i64, _c_i64]),
+    "pk_gate_logits": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p, _c_i64, _p]),
     "pk_route_topk": (_c_int, [_p, _c_i64, _c_i64, _c_i64, _c_int, _c_f32, _p, _p, _p]),
     "pk_route_topk_bwd": (_c_int, [_p, _p, _p, _c_i64, _c_i64, _c_i64, _c_int, _c_f32, _p, _p]),
-    "pk_gate_logits_bwd": (_c_int, [_p, _p, _c_int, _p, _p, _p, _p, _c_int, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_gate_bwd_workspace_bytes": (_c_i64, [_c_i64, _c_i64, _c_i64]),
+    "pk_gate_logits_bwd": (_c_int, [_p, _p, _c_int, _p, _p, _p, _p, _c_int, _c_i64, _c_i64, _c_i64, _p, _c_i64, _p]),
     "pk_sort_workspace_bytes": (_c_i64, [_c_i64, _c_i64]),
     "pk_sort_by_expert": (_c_int, [_p, _c_i64, _c_i64, _p, _p, _p, _p, _p, _c_i64, _p]),
     "pk_counts_to_starts": (_c_int, [_p, _c_int, _c_i64, _p, _p]),

@@ -13,16 +13,16 @@ namespace {
 // ===================================================================== bf16 MFMA path
 namespace mf {
 
-constexpr int BM = 128, BN = 128, BK = 64, THREADS = 256;
-constexpr int LDS_LD = BK + 8;  // bf16 elements per LDS row: 144 B keeps 16-B alignment and
-                                // spreads 16 consecutive rows over all banks for b128 reads
+constexpr int BK = 64, THREADS = 256;
 constexpr int NXCD = 8;
 
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_SWIGLU_BWD = 2 };
 
-__device__ __forceinline__ floatx16_t mfma32(bf16x8_t a, bf16x8_t b, floatx16_t c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
+typedef short shortx4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// 16 zero bytes: the source of operand rows past the end of a ragged reduction range.
+__device__ __attribute__((aligned(16))) const uint32_t g_zero16[4] = {0u, 0u, 0u, 0u};
 
 // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of
 // logical tiles so that tiles sharing operands hit the same L2.  gridDim.x is a multiple of 8.
@@ -31,9 +31,163 @@ __device__ __forceinline__ int logical_block() {
   return (blockIdx.x % NXCD) * per + blockIdx.x / NXCD;
 }
 
+// Direct global->LDS load of 16 bytes per lane: lane l's bytes land at lds_base + 16*l.
+// Issued from inline asm so that the compiler does not serialise later LDS reads behind it;
+// completion is tracked by hand with vmcnt (wait_dma) followed by a workgroup barrier.
+__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off"
+               :: "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr)
+               : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_dma() {
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+__device__ __forceinline__ void block_barrier() {
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+  return (uint32_t)(uintptr_t)(lds_ptr_t)p;
+}
+
+// ---------------------------------------------------------------------------------------------
+// LDS tile layouts.  Both are ROWS*128 bytes; 16-byte chunks are XOR-swizzled so that the
+// fragment reads below touch every bank once.
+//
+// KC tile: [ROWS rows of the M or N index][64 k], k contiguous (128 B per row, 8 chunks).
+//          chunk c of row r sits at position c ^ ((r >> 1) & 7).
+// MN tile: [64 k][COLS of the M or N index], the M/N index contiguous (COLS/8 chunks per row).
+//          chunk c of row k sits at position c ^ ((k & 3) << 2).
+//
+// A wave-level dma16 fills 64 consecutive 16-byte slots; which global chunk a lane fetches is
+// chosen so that the swizzled layout comes out.
+
+// Global element offset (within the operand) of the chunk that lane `lane` of load `G`
+// (G-th group of 64 slots of the tile) must fetch, for a KC tile: returns row and k offset.
+__device__ __forceinline__ void kc_slot(int G, int lane, int& row, int& kofs) {
+  row = G * 8 + (lane >> 3);
+  kofs = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+}
+template <int COLS>
+__device__ __forceinline__ void mn_slot(int G, int lane, int& krow, int& cofs) {
+  constexpr int CPR = COLS / 8;
+  const int slot = G * 64 + lane;
+  krow = slot / CPR;
+  cofs = ((slot % CPR) ^ ((krow & 3) << 2)) * 8;
+}
+
+// MFMA operand fragment (8 bf16 per lane: row lane%32, k = 16*ks + 8*(lane/32) + 0..7).
+__device__ __forceinline__ bf16x8_t frag_kc(const char* tile, int row0, int ks, int lane) {
+  const int r = row0 + (lane & 31);
+  const int c = 2 * ks + (lane >> 5);
+  return *reinterpret_cast<const bf16x8_t*>(tile + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
+}
+// Same fragment out of an MN tile through the transposing LDS read: within 16 lanes, lane i
+// points at 4 consecutive columns of k-row i/4 and receives 4 consecutive k of column i.
+template <int COLS>
+__device__ __forceinline__ bf16x8_t frag_mn(const char* tile, int col0, int ks, int lane) {
+  const int i = lane & 15;
+  const int krow = ks * 16 + 8 * (lane >> 5) + (i >> 2);
+  const int col = col0 + 16 * ((lane >> 4) & 1) + 4 * (i & 3);
+  const int pos = (col >> 3) ^ ((i >> 2) << 2);
+  const char* p = tile + krow * (COLS * 2) + pos * 16 + (col & 7) * 2;
+  const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) shortx4_t*)(p));
+  const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) shortx4_t*)(p + 4 * COLS * 2));
+  typedef short shortx8_t __attribute__((ext_vector_type(8)));
+  shortx8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8_t, v);
+}
+
+// Fragments of one 16-deep k-step for a wave tile of TM x TN MFMA tiles.
+template <int TM, int TN>
+struct Frags {
+  bf16x8_t a[TM];
+  bf16x8_t b[TN];
+};
+template <int TM, int TN, bool A_KC, bool B_KC, int ACOLS, int BCOLS>
+__device__ __forceinline__ void load_frags(Frags<TM, TN>& f, const char* At, const char* Bt,
+                                           int wrow0, int wcol0, int ks, int lane) {
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+    f.a[i] = A_KC ? frag_kc(At, wrow0 + 32 * i, ks, lane) : frag_mn<ACOLS>(At, wrow0 + 32 * i, ks, lane);
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+    f.b[j] = B_KC ? frag_kc(Bt, wcol0 + 32 * j, ks, lane) : frag_mn<BCOLS>(Bt, wcol0 + 32 * j, ks, lane);
+}
+
+// One 64-deep k-tile of MFMAs, software pipelined: the fragments of k-step s+1 are requested
+// from LDS before the MFMAs of k-step s are issued, so the ~90-cycle LDS latency is covered.
+// The operands are passed swapped (B first) so that each lane's accumulator holds 4
+// CONSECUTIVE output columns of ONE output row:
+//   acc[i][j][v] = C[row = 32*i + lane%32][col = 32*j + 8*(v/4) + 4*(lane/32) + v%4]
+template <int TM, int TN, bool A_KC, bool B_KC, int ACOLS, int BCOLS>
+__device__ __forceinline__ void mma_tile(const char* At, const char* Bt, int wrow0, int wcol0,
+                                         floatx16_t (&acc)[TM][TN]) {
+  const int lane = threadIdx.x & 63;
+  Frags<TM, TN> f[2];
+  load_frags<TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[0], At, Bt, wrow0, wcol0, 0, lane);
+#pragma unroll
+  for (int ks = 0; ks < BK / 16; ++ks) {
+    if (ks + 1 < BK / 16)
+      load_frags<TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[(ks + 1) & 1], At, Bt, wrow0, wcol0, ks + 1, lane);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[ks & 1].b[j], f[ks & 1].a[i], acc[i][j], 0, 0, 0);
+  }
+}
+
+__device__ __forceinline__ u32x2_t pack4(float a, float b, float c, float d) {
+  bf16x4_t v;
+  v[0] = (bf16_t)a; v[1] = (bf16_t)b; v[2] = (bf16_t)c; v[3] = (bf16_t)d;
+  return __builtin_bit_cast(u32x2_t, v);
+}
+__device__ __forceinline__ void unpack4(u32x2_t p, float (&f)[4]) {
+  bf16x4_t v = __builtin_bit_cast(bf16x4_t, p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f[i] = (float)v[i];
+}
+
+// Wave-private staging of a [ROWS x COLS] bf16 tile through LDS so that global stores are 16
+// bytes per lane and row-contiguous.  Row stride is COLS*2 + 16 bytes (keeps 16-B alignment).
+template <int COLS>
+struct Stage {
+  static constexpr int LD = COLS * 2 + 16;
+  // a lane deposits 4 consecutive columns of one row
+  __device__ static __forceinline__ void put(char* buf, int row, int col, u32x2_t v) {
+    *reinterpret_cast<u32x2_t*>(buf + row * LD + col * 2) = v;
+  }
+  // copy rows [0, nrows) x COLS of the staged tile to global memory (row stride ldc elements)
+  template <int ROWS>
+  __device__ static __forceinline__ void flush(const char* buf, bf16_t* dst, int64_t ldc, int nrows) {
+    constexpr int LANES_PER_ROW = COLS / 8;        // 16 bytes per lane
+    constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+    const int lane = threadIdx.x & 63;
+    const int lr = lane / LANES_PER_ROW, lc = (lane % LANES_PER_ROW) * 8;
+#pragma unroll
+    for (int r0 = 0; r0 < ROWS; r0 += ROWS_PER_PASS) {
+      const int r = r0 + lr;
+      if (r < nrows) {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(buf + r * LD + lc * 2);
+        *reinterpret_cast<u32x4_t*>(dst + (int64_t)r * ldc + lc) = v;
+      }
+    }
+  }
+};
+// LDS traffic of one wave is ordered by the hardware; this only stops the compiler from
+// moving the staged reads above the writes.
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // Ragged-M tile lookup, done redundantly by every wave (no LDS, no barrier).
 // Expert e owns ceil(cnt_e/BM) * n_tiles units, laid out [n-tile][m-tile] so that neighbouring
 // units share the weight tile.  Returns false when `unit` is past the last real tile.
+template <int BM>
 __device__ __forceinline__ bool locate_ragged_m(const int32_t* __restrict__ starts, int E,
                                                 int n_tiles, int unit, int& e_out, int& mt_out,
                                                 int& nt_out) {
@@ -70,63 +224,6 @@ __device__ __forceinline__ bool locate_ragged_m(const int32_t* __restrict__ star
   return true;
 }
 
-// ---- operand tile loaders.  LDS tiles are always [row (M or N index)][k], k contiguous.
-
-// K-contiguous operand: each thread moves 4 chunks of 8 bf16 (16 B); rows r = (tid>>3) + 32*i.
-struct KContigRegs { u32x4_t v[4]; };
-
-__device__ __forceinline__ void store_kcontig(const KContigRegs& r, bf16_t* lds) {
-  const int row = threadIdx.x >> 3, kc = threadIdx.x & 7;
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-    *reinterpret_cast<u32x4_t*>(lds + (row + 32 * i) * LDS_LD + kc * 8) = r.v[i];
-}
-
-// MN-contiguous operand (global layout [k][mn]): each thread loads an 8(k) x 4(mn) block as
-// eight 8-byte pieces, transposes it in registers and writes four 16-byte LDS rows.
-struct MnContigRegs { u32x2_t v[8]; };
-
-__device__ __forceinline__ void store_mncontig(const MnContigRegs& r, bf16_t* lds) {
-  const int ng = threadIdx.x & 31, kg = threadIdx.x >> 5;
-  u32x4_t out[4];
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    // k = 2c (low half) and k = 2c+1 (high half)
-    out[0][c] = __builtin_amdgcn_perm(r.v[2 * c + 1][0], r.v[2 * c][0], 0x05040100u);
-    out[1][c] = __builtin_amdgcn_perm(r.v[2 * c + 1][0], r.v[2 * c][0], 0x07060302u);
-    out[2][c] = __builtin_amdgcn_perm(r.v[2 * c + 1][1], r.v[2 * c][1], 0x05040100u);
-    out[3][c] = __builtin_amdgcn_perm(r.v[2 * c + 1][1], r.v[2 * c][1], 0x07060302u);
-  }
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-    *reinterpret_cast<u32x4_t*>(lds + (ng * 4 + j) * LDS_LD + kg * 8) = out[j];
-}
-
-// One 64-deep k-tile of MFMAs for this wave's 64x64 sub-tile.
-__device__ __forceinline__ void mma_tile(const bf16_t* As, const bf16_t* Bs, int wm, int wn,
-                                         floatx16_t (&acc)[2][2]) {
-  const int lane = threadIdx.x & 63;
-  const int r = lane & 31, kq = (lane >> 5) * 8;
-#pragma unroll
-  for (int ks = 0; ks < BK / 16; ++ks) {
-    bf16x8_t a[2], b[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-      a[i] = *reinterpret_cast<const bf16x8_t*>(As + (wm * 64 + i * 32 + r) * LDS_LD + ks * 16 + kq);
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-      b[j] = *reinterpret_cast<const bf16x8_t*>(Bs + (wn * 64 + j * 32 + r) * LDS_LD + ks * 16 + kq);
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
-  }
-}
-
-// Accumulator element v of a 32x32 tile held by `lane`: row = 8*(v/4) + 4*(lane/32) + v%4,
-// column = lane%32.
-__device__ __forceinline__ int acc_row(int v, int lane) { return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3); }
-
 struct RaggedMParams {
   const bf16_t* A0;      // A operand of k-segment 0, row-major [rows, lda]
   const bf16_t* A1;      // k-segment 1 (nseg == 2)
@@ -148,144 +245,197 @@ struct RaggedMParams {
   bf16_t* O1;            //            SWIGLU: u;  SWIGLU_BWD: d_u
   bf16_t* O2;            //            SWIGLU: h
   int64_t ldc;
+#ifdef PK_GEMM_DEBUG
+  int32_t debug;         // 1: skip MFMAs, 2: skip loads, 4: skip stores
+#endif
 };
 
-// C[rows_e, N] = A[rows_e, K] . op(B[e])   with B K-contiguous ([N,K], "NT") or
-// MN-contiguous ([K,N], "NN").
-template <bool B_KCONTIG, int EPI>
-__global__ __launch_bounds__(THREADS) void ragged_m_kernel(const RaggedMParams p) {
-  __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_LD];
-  __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS_LD];
+// C[rows_e, N] = A[rows_e, K] . op(B[e]) with B K-contiguous ([N,K]) or MN-contiguous ([K,N]).
+// Block tile BM x BN, WMW x WNW waves, NS-stage LDS ring filled by direct-to-LDS loads.
+// EPI_SWIGLU: the BN tile rows are [32 gate | 32 up | 32 gate | 32 up ...] of BN/2 output
+// columns, so that a lane holds the gate and the up value of the same element.
+template <int BM, int BN, int WMW, int WNW, int NS, bool B_KC, int EPI>
+__global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMParams p) {
+  constexpr int NTHREADS = 64 * WMW * WNW;
+  constexpr int WTM = BM / WMW, WTN = BN / WNW;          // wave tile
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int A_BYTES = BM * 128, STAGE = (BM + BN) * 128;
+  constexpr int LA = BM * 8 / NTHREADS, LB = BN * 8 / NTHREADS;   // dma16 per thread per tile
+  static_assert(LA >= 1 && LB >= 1 && TM >= 1 && TN >= 1, "tile too small for the wave grid");
+  static_assert(EPI != EPI_SWIGLU || (WTN % 64 == 0), "gate/up pairs must stay inside a wave");
+  // output columns a wave writes per output tensor, and its staging buffer
+  constexpr int OUT_COLS = (EPI == EPI_SWIGLU) ? WTN / 2 : WTN;
+  using St = Stage<OUT_COLS>;
+  constexpr int STAGING = WTM * St::LD * (WMW * WNW);
+  constexpr int SMEM = STAGING > NS * STAGE ? STAGING : NS * STAGE;
+  __shared__ __attribute__((aligned(1024))) char smem[SMEM];
 
   int e, mt, nt;
-  if (!locate_ragged_m(p.starts, p.E, p.n_tiles, logical_block(), e, mt, nt)) return;
+  if (!locate_ragged_m<BM>(p.starts, p.E, p.n_tiles, logical_block(), e, mt, nt)) return;
   const int row0 = p.starts[e] + mt * BM;
   const int rows = min(BM, p.starts[e + 1] - row0);
 
-  const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int wm = wave / WNW, wn = wave % WNW;
+  const bool wave_has_rows = wm * WTM < rows;   // waves whose row slice is empty skip the math
 
-  // ---- A loader: rows beyond the expert's range are clamped (their results are not stored)
-  const int ld_r = tid >> 3, ld_kc = tid & 7;
-  int64_t a_off[4];
+  // ---- per-thread source pointers of the dma16 loads (k offset 0 of segment 0)
+  int64_t a_off[LA];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int r = ld_r + 32 * i;
-    r = r < rows ? r : rows - 1;
+  for (int i = 0; i < LA; ++i) {
+    int r, kofs;
+    kc_slot(wave * LA + i, lane, r, kofs);
+    r = r < rows ? r : rows - 1;     // clamp: rows past the expert's range are never stored
     int64_t src = row0 + r;
     if (p.row_map) src = p.row_map[src] / p.map_div;
-    a_off[i] = src * p.lda + ld_kc * 8;
+    a_off[i] = src * p.lda + kofs;
   }
-  // ---- B loader
+  int64_t b_off[LB];
+  int b_mat[LB];
   const int64_t b_base = (int64_t)e * p.strideB;
-  int64_t b_off[4];   // K-contiguous: per-row offsets
-  int b_mat[4];
-  if (B_KCONTIG) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = ld_r + 32 * i;
+  for (int i = 0; i < LB; ++i) {
+    b_mat[i] = 0;
+    if (B_KC) {
+      int r, kofs;
+      kc_slot(wave * LB + i, lane, r, kofs);
       int n;
-      if (EPI == EPI_SWIGLU) {  // LDS rows: 32 gate | 32 up | 32 gate | 32 up
+      if (EPI == EPI_SWIGLU) {
         b_mat[i] = (r >> 5) & 1;
-        n = nt * 64 + (r >> 6) * 32 + (r & 31);
+        n = nt * (BN / 2) + (r >> 6) * 32 + (r & 31);
       } else {
-        b_mat[i] = 0;
         n = nt * BN + r;
       }
-      b_off[i] = b_base + (int64_t)n * p.ldb + ld_kc * 8;
+      b_off[i] = b_base + (int64_t)n * p.ldb + kofs;
+    } else {
+      int krow, cofs;
+      mn_slot<BN>(wave * LB + i, lane, krow, cofs);
+      b_off[i] = b_base + (int64_t)krow * p.ldb + (int64_t)nt * BN + cofs;
     }
   }
-  const int tn_g = tid & 31, tk_g = tid >> 5;  // MN-contiguous: 8(k) x 4(n) block per thread
-
-  floatx16_t acc[2][2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const int kt_per_seg = p.Kseg / BK;
   const int nkt = kt_per_seg * p.nseg;
 
-  KContigRegs a_regs, bk_regs;
-  MnContigRegs bm_regs;
-
-  auto issue_loads = [&](int kt) {
+  auto issue = [&](int kt, int stage) {
+    char* st = smem + stage * STAGE;
     const int seg = kt >= kt_per_seg ? 1 : 0;
     const int k0 = (kt - seg * kt_per_seg) * BK;
     const bf16_t* A = seg ? p.A1 : p.A0;
+    const uint32_t a_lds = lds_addr(st) + (wave * LA) * 1024;
+    const uint32_t b_lds = lds_addr(st + A_BYTES) + (wave * LB) * 1024;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a_regs.v[i] = *reinterpret_cast<const u32x4_t*>(A + a_off[i] + k0);
-    if (B_KCONTIG) {
+    for (int i = 0; i < LA; ++i) dma16(A + a_off[i] + k0, a_lds + i * 1024);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const bf16_t* B = (EPI == EPI_SWIGLU) ? (b_mat[i] ? p.B1 : p.B0) : (seg ? p.B1 : p.B0);
-        bk_regs.v[i] = *reinterpret_cast<const u32x4_t*>(B + b_off[i] + k0);
-      }
-    } else {
-      const bf16_t* B = (seg ? p.B1 : p.B0) + b_base + (int64_t)(k0 + tk_g * 8) * p.ldb +
-                        (int64_t)nt * BN + tn_g * 4;
-#pragma unroll
-      for (int kk = 0; kk < 8; ++kk)
-        bm_regs.v[kk] = *reinterpret_cast<const u32x2_t*>(B + (int64_t)kk * p.ldb);
+    for (int i = 0; i < LB; ++i) {
+      const bf16_t* B = (EPI == EPI_SWIGLU) ? (b_mat[i] ? p.B1 : p.B0) : (seg ? p.B1 : p.B0);
+      dma16(B + b_off[i] + (B_KC ? (int64_t)k0 : (int64_t)k0 * p.ldb), b_lds + i * 1024);
     }
   };
 
-  issue_loads(0);
-  for (int kt = 0; kt < nkt; ++kt) {
-    store_kcontig(a_regs, As);
-    if (B_KCONTIG) store_kcontig(bk_regs, Bs); else store_mncontig(bm_regs, Bs);
-    __syncthreads();
-    if (kt + 1 < nkt) issue_loads(kt + 1);
-    mma_tile(As, Bs, wm, wn, acc);
-    __syncthreads();
-  }
+  floatx16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  // ---- epilogue
-  const int col_in_tile = lane & 31;
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s)
+    if (s < nkt) issue(s, s);
+  int cur = 0;            // stage of tile kt
+  int nxt = NS - 1;       // stage of tile kt + NS - 1
+  for (int kt = 0; kt < nkt; ++kt) {
+    // tile kt has landed once at most the NS-2 younger tiles are still in flight
+    if (kt + NS - 2 < nkt) wait_dma<(NS - 2) * (LA + LB)>(); else wait_dma<0>();
+    block_barrier();   // everyone's part of tile kt is in LDS; everyone is done reading tile kt-1
+#ifdef PK_GEMM_DEBUG
+    if (!(p.debug & 2))
+#endif
+    if (kt + NS - 1 < nkt) issue(kt + NS - 1, nxt);
+    const char* st = smem + cur * STAGE;
+#ifdef PK_GEMM_DEBUG
+    if (!(p.debug & 1))
+#endif
+    if (wave_has_rows)
+      mma_tile<TM, TN, true, B_KC, BM, BN>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
+    cur = cur + 1 == NS ? 0 : cur + 1;
+    nxt = nxt + 1 == NS ? 0 : nxt + 1;
+  }
+#ifdef PK_GEMM_DEBUG
+  if (p.debug & 4) { if (acc[0][0][0] != 12345.678f) return; }
+#endif
+
+  // ---- epilogue: stage each wave's tile through LDS, then 16-byte row-contiguous stores
+  block_barrier();   // the ring is free: every wave has finished its last fragment reads
+  if (!wave_has_rows) return;
+  char* sbuf = smem + wave * (WTM * St::LD);
+  const int lrow = lane & 31, lq = 4 * (lane >> 5);
+  const int wrows = min(WTM, rows - wm * WTM);          // valid rows of this wave's slice
+  const int64_t grow0 = (int64_t)(row0 + wm * WTM) * p.ldc;
   if (EPI == EPI_SWIGLU) {
-    const int64_t col = (int64_t)nt * 64 + wn * 32 + col_in_tile;
+    const int64_t gcol0 = (int64_t)nt * (BN / 2) + wn * OUT_COLS;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int which = 0; which < 3; ++which) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int r = wm * 64 + i * 32 + acc_row(v, lane);
-        if (r < rows) {
-          const bf16_t gb = (bf16_t)acc[i][0][v], ub = (bf16_t)acc[i][1][v];
-          const float g = (float)gb, u = (float)ub;
-          const float h = (g / (1.f + __expf(-g))) * u;
-          const int64_t o = (int64_t)(row0 + r) * p.ldc + col;
-          p.O0[o] = gb;
-          p.O1[o] = ub;
-          p.O2[o] = (bf16_t)h;
-        }
-      }
-  } else {
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+        for (int j = 0; j < TN; j += 2)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int64_t col = (int64_t)nt * BN + wn * 64 + j * 32 + col_in_tile;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int r = wm * 64 + i * 32 + acc_row(v, lane);
-          if (r < rows) {
-            const int64_t o = (int64_t)(row0 + r) * p.ldc + col;
-            if (EPI == EPI_PLAIN) {
-              p.O0[o] = (bf16_t)acc[i][j][v];
-            } else {  // SwiGLU backward: acc = d_h
-              const float dh = (float)(bf16_t)acc[i][j][v];
-              const float g = (float)p.Gin[o], u = (float)p.Uin[o];
-              const float s = 1.f / (1.f + __expf(-g));
-              const float silu = g * s;
-              p.O0[o] = (bf16_t)(dh * u * (s * (1.f + g * (1.f - s))));
-              p.O1[o] = (bf16_t)(dh * silu);
+          for (int q = 0; q < 4; ++q) {
+            const u32x2_t gp = pack4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+            const u32x2_t up = pack4(acc[i][j + 1][4 * q], acc[i][j + 1][4 * q + 1], acc[i][j + 1][4 * q + 2], acc[i][j + 1][4 * q + 3]);
+            u32x2_t v = which == 0 ? gp : up;
+            if (which == 2) {
+              float g[4], u[4];
+              unpack4(gp, g);
+              unpack4(up, u);
+              v = pack4((g[0] / (1.f + __expf(-g[0]))) * u[0], (g[1] / (1.f + __expf(-g[1]))) * u[1],
+                        (g[2] / (1.f + __expf(-g[2]))) * u[2], (g[3] / (1.f + __expf(-g[3]))) * u[3]);
             }
+            St::put(sbuf, 32 * i + lrow, 16 * j + 8 * q + lq, v);
           }
-        }
+      wave_lds_fence();
+      bf16_t* dst = (which == 0 ? p.O0 : which == 1 ? p.O1 : p.O2) + grow0 + gcol0;
+      St::template flush<WTM>(sbuf, dst, p.ldc, wrows);
+      wave_lds_fence();
+    }
+  } else {
+    const int64_t gcol0 = (int64_t)nt * BN + wn * WTN;
+#pragma unroll
+    for (int which = 0; which < (EPI == EPI_PLAIN ? 1 : 2); ++which) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int r = 32 * i + lrow;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int c = 32 * j + 8 * q + lq;
+            u32x2_t v = pack4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+            if (EPI == EPI_SWIGLU_BWD) {   // acc = d_h (rounded to bf16 like the reference's bmm output)
+              float dh[4], g[4], u[4], o[4];
+              unpack4(v, dh);
+              const int rr = r < wrows ? r : wrows - 1;
+              const int64_t off = grow0 + (int64_t)rr * p.ldc + gcol0 + c;
+              unpack4(*reinterpret_cast<const u32x2_t*>(p.Gin + off), g);
+              unpack4(*reinterpret_cast<const u32x2_t*>(p.Uin + off), u);
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                const float sg = 1.f / (1.f + __expf(-g[t]));
+                o[t] = which == 0 ? dh[t] * u[t] * (sg * (1.f + g[t] * (1.f - sg))) : dh[t] * (g[t] * sg);
+              }
+              v = pack4(o[0], o[1], o[2], o[3]);
+            }
+            St::put(sbuf, r, c, v);
+          }
       }
+      wave_lds_fence();
+      bf16_t* dst = (which == 0 ? p.O0 : p.O1) + grow0 + gcol0;
+      St::template flush<WTM>(sbuf, dst, p.ldc, wrows);
+      wave_lds_fence();
+    }
   }
 }
 
@@ -305,26 +455,17 @@ struct WgradParams {
   int32_t tiles_per_expert;  // (M/BM)*(N/BN), identical for the three problems
 };
 
-__device__ __forceinline__ void wgrad_load(MnContigRegs& r, const bf16_t* base, int64_t ld,
-                                           const int32_t* map, int map_div, int row_begin,
-                                           int row_end, int k0, int col0) {
-  const int cg = threadIdx.x & 31, kg = threadIdx.x >> 5;
-#pragma unroll
-  for (int kk = 0; kk < 8; ++kk) {
-    const int row = row_begin + k0 + kg * 8 + kk;
-    u32x2_t v = {0u, 0u};
-    if (row < row_end) {
-      int64_t src = row;
-      if (map) src = map[row] / map_div;
-      v = *reinterpret_cast<const u32x2_t*>(base + src * ld + col0 + cg * 4);
-    }
-    r.v[kk] = v;
-  }
-}
-
-__global__ __launch_bounds__(THREADS) void wgrad_kernel(const WgradParams p) {
-  __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_LD];
-  __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS_LD];
+template <int BM, int BN, int WMW, int WNW, int NS>
+__global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams p) {
+  constexpr int NTHREADS = 64 * WMW * WNW;
+  constexpr int WTM = BM / WMW, WTN = BN / WNW;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int A_BYTES = BM * 128, STAGE = (BM + BN) * 128;
+  constexpr int LA = BM * 8 / NTHREADS, LB = BN * 8 / NTHREADS;
+  using St = Stage<WTN>;
+  constexpr int STAGING = WTM * St::LD * (WMW * WNW);
+  constexpr int SMEM = STAGING > NS * STAGE ? STAGING : NS * STAGE;
+  __shared__ __attribute__((aligned(1024))) char smem[SMEM];
 
   const WgradProblem& q = p.prob[blockIdx.y];
   const int L = logical_block();
@@ -336,61 +477,103 @@ __global__ __launch_bounds__(THREADS) void wgrad_kernel(const WgradParams p) {
   const int row_begin = p.starts[e], row_end = p.starts[e + 1];
   const int nkt = (row_end - row_begin + BK - 1) / BK;
 
-  const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int wm = wave / WNW, wn = wave % WNW;
 
-  floatx16_t acc[2][2];
+  int a_k[LA], a_c[LA], b_k[LB], b_c[LB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < LA; ++i) mn_slot<BM>(wave * LA + i, lane, a_k[i], a_c[i]);
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+  for (int i = 0; i < LB; ++i) mn_slot<BN>(wave * LB + i, lane, b_k[i], b_c[i]);
+
+  auto issue = [&](int kt, int stage) {
+    char* st = smem + stage * STAGE;
+    const uint32_t a_lds = lds_addr(st) + (wave * LA) * 1024;
+    const uint32_t b_lds = lds_addr(st + A_BYTES) + (wave * LB) * 1024;
+    const int k0 = row_begin + kt * BK;
+#pragma unroll
+    for (int i = 0; i < LA; ++i) {
+      const int row = k0 + a_k[i];
+      const void* src = g_zero16;
+      if (row < row_end) {
+        int64_t r = row;
+        if (q.a_map) r = q.a_map[row] / p.map_div;
+        src = q.A + r * q.lda + (int64_t)mt * BM + a_c[i];
+      }
+      dma16(src, a_lds + i * 1024);
+    }
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+      const int row = k0 + b_k[i];
+      const void* src = g_zero16;
+      if (row < row_end) {
+        int64_t r = row;
+        if (q.b_map) r = q.b_map[row] / p.map_div;
+        src = q.B + r * q.ldb + (int64_t)nt * BN + b_c[i];
+      }
+      dma16(src, b_lds + i * 1024);
+    }
+  };
+
+  floatx16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  MnContigRegs a_regs, b_regs;
-  if (nkt > 0) {
-    wgrad_load(a_regs, q.A, q.lda, q.a_map, p.map_div, row_begin, row_end, 0, mt * BM);
-    wgrad_load(b_regs, q.B, q.ldb, q.b_map, p.map_div, row_begin, row_end, 0, nt * BN);
-  }
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s)
+    if (s < nkt) issue(s, s);
+  int cur = 0, nxt = NS - 1;
   for (int kt = 0; kt < nkt; ++kt) {
-    store_mncontig(a_regs, As);
-    store_mncontig(b_regs, Bs);
-    __syncthreads();
-    if (kt + 1 < nkt) {
-      wgrad_load(a_regs, q.A, q.lda, q.a_map, p.map_div, row_begin, row_end, (kt + 1) * BK, mt * BM);
-      wgrad_load(b_regs, q.B, q.ldb, q.b_map, p.map_div, row_begin, row_end, (kt + 1) * BK, nt * BN);
-    }
-    mma_tile(As, Bs, wm, wn, acc);
-    __syncthreads();
+    if (kt + NS - 2 < nkt) wait_dma<(NS - 2) * (LA + LB)>(); else wait_dma<0>();
+    block_barrier();
+    if (kt + NS - 1 < nkt) issue(kt + NS - 1, nxt);
+    const char* st = smem + cur * STAGE;
+    mma_tile<TM, TN, false, false, BM, BN>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
+    cur = cur + 1 == NS ? 0 : cur + 1;
+    nxt = nxt + 1 == NS ? 0 : nxt + 1;
   }
 
-  bf16_t* C = q.C + (int64_t)e * q.M * q.N;
-  const int col_in_tile = lane & 31;
+  block_barrier();
+  bf16_t* C = q.C + (int64_t)e * q.M * q.N + ((int64_t)mt * BM + wm * WTM) * q.N + (int64_t)nt * BN + wn * WTN;
+  char* sbuf = smem + wave * (WTM * St::LD);
+  const int lrow = lane & 31, lq = 4 * (lane >> 5);
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i) {
+    const int r = 32 * i + lrow;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int64_t col = (int64_t)nt * BN + wn * 64 + j * 32 + col_in_tile;
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int64_t r = (int64_t)mt * BM + wm * 64 + i * 32 + acc_row(v, lane);
-        const int64_t o = r * q.N + col;
-        float val = acc[i][j][v];
-        if (p.accumulate) val += (float)C[o];
-        C[o] = (bf16_t)val;
+      for (int qd = 0; qd < 4; ++qd) {
+        const int c = 32 * j + 8 * qd + lq;
+        float v[4] = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
+        if (p.accumulate) {
+          float old[4];
+          unpack4(*reinterpret_cast<const u32x2_t*>(C + (int64_t)r * q.N + c), old);
+#pragma unroll
+          for (int t2 = 0; t2 < 4; ++t2) v[t2] += old[t2];
+        }
+        St::put(sbuf, r, c, pack4(v[0], v[1], v[2], v[3]));
       }
-    }
+  }
+  wave_lds_fence();
+  St::template flush<WTM>(sbuf, C, q.N, WTM);
 }
 
 inline int round_up_xcd(int64_t n) { return (int)(pk_ceil_div(n, NXCD) * NXCD); }
 
-template <bool B_KCONTIG, int EPI>
+template <int BM, int BN, int WMW, int WNW, int NS, bool B_KC, int EPI>
 int launch_ragged_m(RaggedMParams p, int64_t A_rows, int kernel_id, hipStream_t s) {
+#ifdef PK_GEMM_DEBUG
+  { const char* d = getenv("PK_GEMM_DEBUG_MODE"); p.debug = d ? atoi(d) : 0; }
+#endif
   const int64_t max_units = (pk_ceil_div(A_rows, BM) + p.E) * p.n_tiles;
   if (max_units > 0x7ffffff0ll) return PK_ERR_SHAPE;
-  PK_LAUNCH_NOCHECK(kernel_id, s, (ragged_m_kernel<B_KCONTIG, EPI>), dim3(round_up_xcd(max_units)),
-                     dim3(THREADS), 0, s, p);
+  PK_LAUNCH_NOCHECK(kernel_id, s, (ragged_m_kernel<BM, BN, WMW, WNW, NS, B_KC, EPI>),
+                    dim3(round_up_xcd(max_units)), dim3(64 * WMW * WNW), 0, s, p);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
 }
@@ -450,6 +633,14 @@ int simt_ragged_k(const void* A, int64_t lda, const int32_t* a_map, const void* 
   p.gA = 0; p.gB = 0; p.gC = M * N;
   return pk_simt::launch<T, T, T>(p, s);
 }
+
+// Tile configurations: BM, BN, waves along M, waves along N, LDS stages.
+#define PK_RM_BIG 128, 256, 2, 4, 3     /* 8 waves, 64x64 wave tiles, 144 KB ring */
+#define PK_RM_SMALL 128, 128, 2, 2, 3   /* 4 waves, 64x64 wave tiles,  96 KB ring */
+#define PK_WG_BIG 256, 256, 2, 2, 2     /* 4 waves, 128x128 wave tiles, 128 KB ring */
+#define PK_WG_BIG_THREADS 256
+#define PK_WG_SMALL 128, 128, 2, 2, 3
+#define PK_WG_SMALL_THREADS 256
 
 bool mfma_shape_ok(int64_t H, int64_t I) { return H % 128 == 0 && I % 128 == 0; }
 
@@ -537,18 +728,22 @@ int pk_grouped_swiglu_fwd(const void* x_rows, const int32_t* row_map, int64_t ro
   p.row_map = row_map; p.map_div = (int32_t)row_map_div;
   p.B0 = (const bf16_t*)w1; p.B1 = (const bf16_t*)w3; p.ldb = H; p.strideB = I * H;
   p.starts = starts; p.E = (int32_t)E; p.Kseg = (int32_t)H; p.nseg = 1;
-  p.n_tiles = (int32_t)(I / 64);
   p.O0 = (bf16_t*)g; p.O1 = (bf16_t*)u; p.O2 = (bf16_t*)h; p.ldc = I;
-  rc = mf::launch_ragged_m<true, mf::EPI_SWIGLU>(p, A, pk_timing::K_SWIGLU_GATE_UP, s);
+  p.n_tiles = (int32_t)(I / 128);   // a 256-row weight tile = 128 gate + 128 up columns
+  rc = mf::launch_ragged_m<PK_RM_BIG, true, mf::EPI_SWIGLU>(p, A, pk_timing::K_SWIGLU_GATE_UP, s);
   if (rc) return rc;
 
   mf::RaggedMParams q = {};
   q.A0 = (const bf16_t*)h; q.lda = I;
   q.B0 = (const bf16_t*)w2; q.B1 = nullptr; q.ldb = I; q.strideB = H * I;
   q.starts = starts; q.E = (int32_t)E; q.Kseg = (int32_t)I; q.nseg = 1;
-  q.n_tiles = (int32_t)(H / mf::BN);
   q.O0 = (bf16_t*)y; q.ldc = H;
-  return mf::launch_ragged_m<true, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DOWN, s);
+  if (H % 256 == 0) {
+    q.n_tiles = (int32_t)(H / 256);
+    return mf::launch_ragged_m<PK_RM_BIG, true, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DOWN, s);
+  }
+  q.n_tiles = (int32_t)(H / 128);
+  return mf::launch_ragged_m<PK_RM_SMALL, true, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DOWN, s);
 }
 
 int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, const void* w3,
@@ -571,10 +766,15 @@ int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, con
   p.A0 = (const bf16_t*)d_y; p.lda = H;
   p.B0 = (const bf16_t*)w2; p.ldb = I; p.strideB = H * I;
   p.starts = starts; p.E = (int32_t)E; p.Kseg = (int32_t)H; p.nseg = 1;
-  p.n_tiles = (int32_t)(I / mf::BN);
   p.Gin = (const bf16_t*)g; p.Uin = (const bf16_t*)u;
   p.O0 = (bf16_t*)d_g; p.O1 = (bf16_t*)d_u; p.ldc = I;
-  rc = mf::launch_ragged_m<false, mf::EPI_SWIGLU_BWD>(p, A, pk_timing::K_SWIGLU_DGRAD_DH, s);
+  if (I % 256 == 0) {
+    p.n_tiles = (int32_t)(I / 256);
+    rc = mf::launch_ragged_m<PK_RM_BIG, false, mf::EPI_SWIGLU_BWD>(p, A, pk_timing::K_SWIGLU_DGRAD_DH, s);
+  } else {
+    p.n_tiles = (int32_t)(I / 128);
+    rc = mf::launch_ragged_m<PK_RM_SMALL, false, mf::EPI_SWIGLU_BWD>(p, A, pk_timing::K_SWIGLU_DGRAD_DH, s);
+  }
   if (rc) return rc;
 
   // d_x = [d_g | d_u] . [w1[e] ; w3[e]]
@@ -582,9 +782,13 @@ int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, con
   q.A0 = (const bf16_t*)d_g; q.A1 = (const bf16_t*)d_u; q.lda = I;
   q.B0 = (const bf16_t*)w1; q.B1 = (const bf16_t*)w3; q.ldb = H; q.strideB = I * H;
   q.starts = starts; q.E = (int32_t)E; q.Kseg = (int32_t)I; q.nseg = 2;
-  q.n_tiles = (int32_t)(H / mf::BN);
   q.O0 = (bf16_t*)d_x_sorted; q.ldc = H;
-  return mf::launch_ragged_m<false, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DGRAD_DX, s);
+  if (H % 256 == 0) {
+    q.n_tiles = (int32_t)(H / 256);
+    return mf::launch_ragged_m<PK_RM_BIG, false, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DGRAD_DX, s);
+  }
+  q.n_tiles = (int32_t)(H / 128);
+  return mf::launch_ragged_m<PK_RM_SMALL, false, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DGRAD_DX, s);
 }
 
 int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, const void* d_u,
@@ -629,10 +833,15 @@ int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, con
   if (n == 0) return PK_OK;
   p.starts = starts; p.E = (int32_t)E; p.map_div = (int32_t)row_map_div;
   p.accumulate = accumulate ? 1 : 0;
-  p.tiles_per_expert = (int32_t)((H / mf::BM) * (I / mf::BN));
+  const bool big = (H % 256 == 0) && (I % 256 == 0);
+  const int tile = big ? 256 : 128;
+  p.tiles_per_expert = (int32_t)((H / tile) * (I / tile));
   const int64_t blocks = (int64_t)p.tiles_per_expert * E;
   if (blocks > 0x7ffffff0ll) return PK_ERR_SHAPE;
-  PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_WGRAD, s, mf::wgrad_kernel, dim3(mf::round_up_xcd(blocks), n), dim3(mf::THREADS), 0, s, p);
+  if (big)
+    PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_WGRAD, s, (mf::wgrad_kernel<PK_WG_BIG>), dim3(mf::round_up_xcd(blocks), n), dim3(PK_WG_BIG_THREADS), 0, s, p);
+  else
+    PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_WGRAD, s, (mf::wgrad_kernel<PK_WG_SMALL>), dim3(mf::round_up_xcd(blocks), n), dim3(PK_WG_SMALL_THREADS), 0, s, p);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
 }

@@ -1,6 +1,6 @@
 // Routing: gate logits, wavefront softmax/top-k (+ backward), stable counting sort by expert.
 #include "pk_common.h"
-#include "simt_gemm.h"
+#include "mfma_f32_gemm.h"
 
 namespace {
 
@@ -261,12 +261,6 @@ __global__ __launch_bounds__(1024) void counts_to_starts_kernel(const void* __re
 }
 
 // ------------------------------------------------------------------ small helpers
-__global__ void bias_fill_kernel(float* __restrict__ logits, const float* __restrict__ bias,
-                                 int64_t T, int E) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < T * E) logits[i] = bias[i % E];
-}
-
 // d_bias[e] (+)= sum_t d_logits[t,e]; one block per expert
 __global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ d_logits, int64_t T,
                                                      int E, float* __restrict__ d_bias,
@@ -297,54 +291,104 @@ const char* pk_status_string(int status) {
   }
 }
 
+static int gate_fwd_splits(int64_t H) {
+  int64_t sp = H / 512;
+  return (int)(sp < 1 ? 1 : (sp > 4 ? 4 : sp));
+}
+
+int64_t pk_gate_workspace_bytes(int64_t T, int64_t H, int64_t E) {
+  if (T < 0 || H <= 0 || E <= 0) return PK_ERR_ARG;
+  const int sp = gate_fwd_splits(H);
+  return sp > 1 ? (int64_t)sp * T * E * (int64_t)sizeof(float) : 0;
+}
+
 int pk_gate_logits(const void* x, int x_dtype, const float* w_gate, const float* gate_bias,
-                   float* logits, int64_t T, int64_t H, int64_t E, pk_stream_t stream) {
+                   float* logits, int64_t T, int64_t H, int64_t E, void* workspace,
+                   int64_t workspace_bytes, pk_stream_t stream) {
   if (T < 0 || H <= 0 || E <= 0 || !pk_dtype_ok(x_dtype)) return PK_ERR_ARG;
   if (T == 0) return PK_OK;
   if (!x || !w_gate || !logits) return PK_ERR_ARG;
-  if (T * E > 0x7fffffffll) return PK_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
-  if (gate_bias) {
+  int sp = gate_fwd_splits(H);
+  if (sp > 1 && (!workspace || workspace_bytes < pk_gate_workspace_bytes(T, H, E))) sp = 1;
+  pk_f32mm::Params p = {};
+  p.A = x; p.B = w_gate;
+  p.C = sp > 1 ? reinterpret_cast<float*>(workspace) : logits;
+  p.bias = sp > 1 ? nullptr : gate_bias;
+  p.M = T; p.N = E; p.K = H;
+  p.sam = H; p.sak = 1; p.sbk = 1; p.sbn = H;
+  p.splits = sp; p.accumulate = 0;
+  int rc;
+  if (E > 64) {  // 64-token x 128-expert tiles, 8 waves
+    rc = x_dtype == PK_BF16
+             ? pk_f32mm::launch<2, 4, true, true, bf16_t, float>(p, pk_timing::K_GATE_LOGITS, s)
+             : pk_f32mm::launch<2, 4, true, true, float, float>(p, pk_timing::K_GATE_LOGITS, s);
+  } else {       // 64-token x 64-expert tiles, 4 waves
+    rc = x_dtype == PK_BF16
+             ? pk_f32mm::launch<2, 2, true, true, bf16_t, float>(p, pk_timing::K_GATE_LOGITS, s)
+             : pk_f32mm::launch<2, 2, true, true, float, float>(p, pk_timing::K_GATE_LOGITS, s);
+  }
+  if (rc != PK_OK) return rc;
+  if (sp > 1) {
     const int64_t n = T * E;
-    PK_LAUNCH_NOCHECK(pk_timing::K_MISC, s, bias_fill_kernel, dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
-                       logits, gate_bias, T, (int)E);
+    PK_LAUNCH_NOCHECK(pk_timing::K_GATE_LOGITS, s, pk_f32mm::reduce_partials_kernel,
+                      dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
+                      reinterpret_cast<const float*>(workspace), logits, n, sp, 0, gate_bias, (int)E);
     PK_RETURN_IF_LAUNCH_FAILED();
   }
-  pk_simt::Params p = {};
-  p.A = x; p.B = w_gate; p.C = logits;
-  p.ragged = pk_simt::RAGGED_NONE; p.G = 1; p.accumulate = gate_bias ? 1 : 0;
-  p.M = T; p.N = E; p.K = H;
-  p.sam = H; p.sak = 1; p.sbk = 1; p.sbn = H; p.scm = E; p.scn = 1;
-  return x_dtype == PK_BF16 ? pk_simt::launch<bf16_t, float, float>(p, s)
-                            : pk_simt::launch<float, float, float>(p, s);
+  return PK_OK;
+}
+
+static int gate_bwd_splits(int64_t T) {
+  int64_t sp = T / 512;
+  return (int)(sp < 1 ? 1 : (sp > 8 ? 8 : sp));
+}
+
+int64_t pk_gate_bwd_workspace_bytes(int64_t T, int64_t H, int64_t E) {
+  if (T < 0 || H <= 0 || E <= 0) return PK_ERR_ARG;
+  const int sp = gate_bwd_splits(T);
+  return sp > 1 ? (int64_t)sp * E * H * (int64_t)sizeof(float) : 0;
 }
 
 int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const float* w_gate,
                        float* d_x_f32, float* d_w_gate, float* d_gate_bias, int accumulate,
-                       int64_t T, int64_t H, int64_t E, pk_stream_t stream) {
+                       int64_t T, int64_t H, int64_t E, void* workspace, int64_t workspace_bytes,
+                       pk_stream_t stream) {
   if (T < 0 || H <= 0 || E <= 0 || !pk_dtype_ok(x_dtype)) return PK_ERR_ARG;
   if (!d_logits && T > 0) return PK_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   if (d_x_f32 && T > 0) {
     if (!w_gate) return PK_ERR_ARG;
-    pk_simt::Params p = {};
+    pk_f32mm::Params p = {};
     p.A = d_logits; p.B = w_gate; p.C = d_x_f32;
-    p.ragged = pk_simt::RAGGED_NONE; p.G = 1; p.accumulate = 0;
     p.M = T; p.N = H; p.K = E;
-    p.sam = E; p.sak = 1; p.sbk = H; p.sbn = 1; p.scm = H; p.scn = 1;
-    int rc = pk_simt::launch<float, float, float>(p, s);
+    p.sam = E; p.sak = 1; p.sbk = H; p.sbn = 1;
+    p.splits = 1; p.accumulate = 0;
+    int rc = pk_f32mm::launch<2, 2, true, false, float, float>(p, pk_timing::K_GATE_LOGITS_BWD, s);
     if (rc != PK_OK) return rc;
   }
   if (d_w_gate) {
     if (!x && T > 0) return PK_ERR_ARG;
-    pk_simt::Params p = {};
-    p.A = d_logits; p.B = x; p.C = d_w_gate;
-    p.ragged = pk_simt::RAGGED_NONE; p.G = 1; p.accumulate = accumulate ? 1 : 0;
+    int sp = gate_bwd_splits(T);
+    if (sp > 1 && (!workspace || workspace_bytes < pk_gate_bwd_workspace_bytes(T, H, E))) sp = 1;
+    pk_f32mm::Params p = {};
+    p.A = d_logits; p.B = x;
+    p.C = sp > 1 ? reinterpret_cast<float*>(workspace) : d_w_gate;
     p.M = E; p.N = H; p.K = T;
-    p.sam = 1; p.sak = E; p.sbk = H; p.sbn = 1; p.scm = H; p.scn = 1;
-    int rc = x_dtype == PK_BF16 ? pk_simt::launch<float, bf16_t, float>(p, s)
-                                : pk_simt::launch<float, float, float>(p, s);
+    p.sam = 1; p.sak = E; p.sbk = H; p.sbn = 1;
+    p.splits = sp; p.accumulate = (sp == 1 && accumulate) ? 1 : 0;
+    int rc = x_dtype == PK_BF16
+                 ? pk_f32mm::launch<2, 2, false, false, float, bf16_t>(p, pk_timing::K_GATE_LOGITS_BWD, s)
+                 : pk_f32mm::launch<2, 2, false, false, float, float>(p, pk_timing::K_GATE_LOGITS_BWD, s);
     if (rc != PK_OK) return rc;
+    if (sp > 1) {
+      const int64_t n = E * H;
+      PK_LAUNCH_NOCHECK(pk_timing::K_GATE_LOGITS_BWD, s, pk_f32mm::reduce_partials_kernel,
+                        dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
+                        reinterpret_cast<const float*>(workspace), d_w_gate, n, sp, accumulate ? 1 : 0,
+                        (const float*)nullptr, 1);
+      PK_RETURN_IF_LAUNCH_FAILED();
+    }
   }
   if (d_gate_bias) {
     PK_LAUNCH_NOCHECK(pk_timing::K_MISC, s, colsum_kernel, dim3((unsigned)E), dim3(256), 0, s, d_logits, T, (int)E,

@@ -33,8 +33,10 @@ def gate_logits(x: torch.Tensor, w_gate: torch.Tensor, gate_bias: torch.Tensor |
         _check(gate_bias.dtype == torch.float32 and gate_bias.shape == (E,), "gate_logits: bias must be float32 [E]")
     x = x.contiguous()
     logits = torch.empty((T, E), dtype=torch.float32, device=x.device)
+    ws_bytes = int(_lib.load().pk_gate_workspace_bytes(T, H, E))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes > 0 else None
     call("pk_gate_logits", ptr(x), dtype_code(x.dtype), ptr(w_gate.contiguous()), ptr(gate_bias), ptr(logits),
-         T, H, E, current_stream(x.device))
+         T, H, E, ptr(ws), ws_bytes if ws is not None else 0, current_stream(x.device))
     return logits
 
 
@@ -44,8 +46,14 @@ def gate_logits_bwd(d_logits, x, w_gate, need_dx=True, d_w_gate=None, d_gate_bia
     T, E = d_logits.shape
     H = x.shape[1]
     d_x = torch.empty((T, H), dtype=torch.float32, device=x.device) if need_dx else None
+    ws = None
+    if d_w_gate is not None:
+        ws_bytes = int(_lib.load().pk_gate_bwd_workspace_bytes(T, H, E))
+        if ws_bytes > 0:
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
     call("pk_gate_logits_bwd", ptr(d_logits.contiguous()), ptr(x.contiguous()), dtype_code(x.dtype), ptr(w_gate.contiguous()),
-         ptr(d_x), ptr(d_w_gate), ptr(d_gate_bias), int(bool(accumulate)), T, H, E, current_stream(x.device))
+         ptr(d_x), ptr(d_w_gate), ptr(d_gate_bias), int(bool(accumulate)), T, H, E, ptr(ws),
+         0 if ws is None else ws.numel(), current_stream(x.device))
     return d_x
 
 
