@@ -19,6 +19,10 @@ constexpr int NXCD = 8;
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_SWIGLU_BWD = 2 };
 
 typedef short shortx4_t __attribute__((ext_vector_type(4)));
+// Read-only tables (row offsets, row maps) addressed wave-uniformly: going through the constant
+// address space makes these scalar loads (lgkmcnt), which leaves vmcnt to the LDS ring.
+typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+__device__ __forceinline__ const_i32_ptr as_const(const int32_t* p) { return (const_i32_ptr)(uintptr_t)p; }
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 // 16 zero bytes: the source of operand rows past the end of a ragged reduction range.
@@ -117,25 +121,55 @@ __device__ __forceinline__ void load_frags(Frags<TM, TN>& f, const char* At, con
 }
 
 // One 64-deep k-tile of MFMAs, software pipelined: the fragments of k-step s+1 are requested
-// from LDS before the MFMAs of k-step s are issued, so the ~90-cycle LDS latency is covered.
+// from LDS before / while the MFMAs of k-step s are issued, so the ~90-cycle LDS latency is
+// covered.  LEAN keeps a single copy of the A fragments and refills each one right after its
+// last use (fewer registers, for the 128x128 wave tiles).
 // The operands are passed swapped (B first) so that each lane's accumulator holds 4
 // CONSECUTIVE output columns of ONE output row:
 //   acc[i][j][v] = C[row = 32*i + lane%32][col = 32*j + 8*(v/4) + 4*(lane/32) + v%4]
-template <int TM, int TN, bool A_KC, bool B_KC, int ACOLS, int BCOLS>
+template <int TM, int TN, bool A_KC, bool B_KC, int ACOLS, int BCOLS, bool LEAN>
 __device__ __forceinline__ void mma_tile(const char* At, const char* Bt, int wrow0, int wcol0,
                                          floatx16_t (&acc)[TM][TN]) {
   const int lane = threadIdx.x & 63;
-  Frags<TM, TN> f[2];
-  load_frags<TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[0], At, Bt, wrow0, wcol0, 0, lane);
-#pragma unroll
-  for (int ks = 0; ks < BK / 16; ++ks) {
-    if (ks + 1 < BK / 16)
-      load_frags<TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[(ks + 1) & 1], At, Bt, wrow0, wcol0, ks + 1, lane);
+  constexpr int KS = BK / 16;
+  if (LEAN) {
+    bf16x8_t a[TM], b[2][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
+      a[i] = A_KC ? frag_kc(At, wrow0 + 32 * i, 0, lane) : frag_mn<ACOLS>(At, wrow0 + 32 * i, 0, lane);
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[ks & 1].b[j], f[ks & 1].a[i], acc[i][j], 0, 0, 0);
+    for (int j = 0; j < TN; ++j)
+      b[0][j] = B_KC ? frag_kc(Bt, wcol0 + 32 * j, 0, lane) : frag_mn<BCOLS>(Bt, wcol0 + 32 * j, 0, lane);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 1 < KS) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          b[(ks + 1) & 1][j] = B_KC ? frag_kc(Bt, wcol0 + 32 * j, ks + 1, lane)
+                                    : frag_mn<BCOLS>(Bt, wcol0 + 32 * j, ks + 1, lane);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[ks & 1][j], a[i], acc[i][j], 0, 0, 0);
+        if (ks + 1 < KS)
+          a[i] = A_KC ? frag_kc(At, wrow0 + 32 * i, ks + 1, lane) : frag_mn<ACOLS>(At, wrow0 + 32 * i, ks + 1, lane);
+      }
+    }
+  } else {
+    Frags<TM, TN> f[2];
+    load_frags<TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[0], At, Bt, wrow0, wcol0, 0, lane);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 1 < KS)
+        load_frags<TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[(ks + 1) & 1], At, Bt, wrow0, wcol0, ks + 1, lane);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[ks & 1].b[j], f[ks & 1].a[i], acc[i][j], 0, 0, 0);
+    }
   }
 }
 
@@ -159,19 +193,29 @@ struct Stage {
   __device__ static __forceinline__ void put(char* buf, int row, int col, u32x2_t v) {
     *reinterpret_cast<u32x2_t*>(buf + row * LD + col * 2) = v;
   }
-  // copy rows [0, nrows) x COLS of the staged tile to global memory (row stride ldc elements)
-  template <int ROWS>
+  // copy rows [0, nrows) x COLS of the staged tile to global memory (row stride ldc elements);
+  // ACC adds the tile to what is already there (fp32 add, one rounding of the sum).
+  template <int ROWS, bool ACC = false>
   __device__ static __forceinline__ void flush(const char* buf, bf16_t* dst, int64_t ldc, int nrows) {
     constexpr int LANES_PER_ROW = COLS / 8;        // 16 bytes per lane
     constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
     const int lane = threadIdx.x & 63;
     const int lr = lane / LANES_PER_ROW, lc = (lane % LANES_PER_ROW) * 8;
-#pragma unroll
+#pragma unroll 4
     for (int r0 = 0; r0 < ROWS; r0 += ROWS_PER_PASS) {
       const int r = r0 + lr;
       if (r < nrows) {
-        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(buf + r * LD + lc * 2);
-        *reinterpret_cast<u32x4_t*>(dst + (int64_t)r * ldc + lc) = v;
+        u32x4_t v = *reinterpret_cast<const u32x4_t*>(buf + r * LD + lc * 2);
+        u32x4_t* g = reinterpret_cast<u32x4_t*>(dst + (int64_t)r * ldc + lc);
+        if (ACC) {
+          const bf16x8_t a = __builtin_bit_cast(bf16x8_t, v);
+          const bf16x8_t o = __builtin_bit_cast(bf16x8_t, *g);
+          bf16x8_t sum;
+#pragma unroll
+          for (int t = 0; t < 8; ++t) sum[t] = (bf16_t)((float)a[t] + (float)o[t]);
+          v = __builtin_bit_cast(u32x4_t, sum);
+        }
+        *g = v;
       }
     }
   }
@@ -359,7 +403,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     if (!(p.debug & 1))
 #endif
     if (wave_has_rows)
-      mma_tile<TM, TN, true, B_KC, BM, BN>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
+      mma_tile<TM, TN, true, B_KC, BM, BN, false>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
     cur = cur + 1 == NS ? 0 : cur + 1;
     nxt = nxt + 1 == NS ? 0 : nxt + 1;
   }
@@ -453,6 +497,9 @@ struct WgradParams {
   int32_t map_div;
   int32_t accumulate;
   int32_t tiles_per_expert;  // (M/BM)*(N/BN), identical for the three problems
+#ifdef PK_GEMM_DEBUG
+  int32_t debug;
+#endif
 };
 
 template <int BM, int BN, int WMW, int WNW, int NS>
@@ -468,23 +515,32 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
   __shared__ __attribute__((aligned(1024))) char smem[SMEM];
 
   const WgradProblem& q = p.prob[blockIdx.y];
-  const int L = logical_block();
-  const int e = L / p.tiles_per_expert;
+  // Experts are dealt round-robin to the 8 XCDs (workgroup b runs on XCD b % 8); the tiles of one
+  // expert stay on one XCD, back to back, so its rows are read from HBM once.
+  const int xcd = blockIdx.x % NXCD, pos = blockIdx.x / NXCD;
+  const int e = xcd + NXCD * (pos / p.tiles_per_expert);
   if (e >= p.E) return;
-  const int t = L % p.tiles_per_expert;
+  const int t = pos % p.tiles_per_expert;
   const int n_tiles = q.N / BN;
   const int mt = t / n_tiles, nt = t % n_tiles;
-  const int row_begin = p.starts[e], row_end = p.starts[e + 1];
+  const const_i32_ptr starts = as_const(p.starts);
+  const int row_begin = starts[e], row_end = starts[e + 1];
   const int nkt = (row_end - row_begin + BK - 1) / BK;
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WNW, wn = wave % WNW;
 
-  int a_k[LA], a_c[LA], b_k[LB], b_c[LB];
-#pragma unroll
-  for (int i = 0; i < LA; ++i) mn_slot<BM>(wave * LA + i, lane, a_k[i], a_c[i]);
-#pragma unroll
-  for (int i = 0; i < LB; ++i) mn_slot<BN>(wave * LB + i, lane, b_k[i], b_c[i]);
+  // One dma16 covers 64 consecutive 16-byte slots = RPI rows of the tile; the row index (and the
+  // optional gather through a row map) is wave-uniform per row, so it is resolved with scalar
+  // loads, which do not disturb the vmcnt bookkeeping of the LDS ring.
+  constexpr int A_CPR = BM / 8, B_CPR = BN / 8;
+  constexpr int A_RPI = 64 / A_CPR, B_RPI = 64 / B_CPR;
+  const const_i32_ptr a_map = as_const(q.a_map), b_map = as_const(q.b_map);
+  const bf16_t* const Abase = q.A + (int64_t)mt * BM;
+  const bf16_t* const Bbase = q.B + (int64_t)nt * BN;
+  const int64_t lda = q.lda, ldb = q.ldb;
+  const int map_div = p.map_div;
 
   auto issue = [&](int kt, int stage) {
     char* st = smem + stage * STAGE;
@@ -493,23 +549,35 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
     const int k0 = row_begin + kt * BK;
 #pragma unroll
     for (int i = 0; i < LA; ++i) {
-      const int row = k0 + a_k[i];
+      int krow, cofs;
+      mn_slot<BM>(wave * LA + i, lane, krow, cofs);
       const void* src = g_zero16;
-      if (row < row_end) {
-        int64_t r = row;
-        if (q.a_map) r = q.a_map[row] / p.map_div;
-        src = q.A + r * q.lda + (int64_t)mt * BM + a_c[i];
+#pragma unroll
+      for (int r = 0; r < A_RPI; ++r) {
+        const int row = k0 + (wave * LA + i) * A_RPI + r;     // wave-uniform
+        if (row < row_end) {
+          int64_t rr = row;
+          if (a_map) rr = a_map[row] / map_div;
+          const bf16_t* cand = Abase + rr * lda;
+          if (lane / A_CPR == r) src = cand + cofs;
+        }
       }
       dma16(src, a_lds + i * 1024);
     }
 #pragma unroll
     for (int i = 0; i < LB; ++i) {
-      const int row = k0 + b_k[i];
+      int krow, cofs;
+      mn_slot<BN>(wave * LB + i, lane, krow, cofs);
       const void* src = g_zero16;
-      if (row < row_end) {
-        int64_t r = row;
-        if (q.b_map) r = q.b_map[row] / p.map_div;
-        src = q.B + r * q.ldb + (int64_t)nt * BN + b_c[i];
+#pragma unroll
+      for (int r = 0; r < B_RPI; ++r) {
+        const int row = k0 + (wave * LB + i) * B_RPI + r;
+        if (row < row_end) {
+          int64_t rr = row;
+          if (b_map) rr = b_map[row] / map_div;
+          const bf16_t* cand = Bbase + rr * ldb;
+          if (lane / B_CPR == r) src = cand + cofs;
+        }
       }
       dma16(src, b_lds + i * 1024);
     }
@@ -530,37 +598,37 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
   for (int kt = 0; kt < nkt; ++kt) {
     if (kt + NS - 2 < nkt) wait_dma<(NS - 2) * (LA + LB)>(); else wait_dma<0>();
     block_barrier();
+#ifdef PK_GEMM_DEBUG
+    if (!(p.debug & 2))
+#endif
     if (kt + NS - 1 < nkt) issue(kt + NS - 1, nxt);
     const char* st = smem + cur * STAGE;
-    mma_tile<TM, TN, false, false, BM, BN>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
+#ifdef PK_GEMM_DEBUG
+    if (!(p.debug & 1))
+#endif
+    mma_tile<TM, TN, false, false, BM, BN, (TM * TN >= 16)>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
     cur = cur + 1 == NS ? 0 : cur + 1;
     nxt = nxt + 1 == NS ? 0 : nxt + 1;
   }
 
+#ifdef PK_GEMM_DEBUG
+  if (p.debug & 4) { if (acc[0][0][0] != 12345.678f) return; }
+#endif
   block_barrier();
   bf16_t* C = q.C + (int64_t)e * q.M * q.N + ((int64_t)mt * BM + wm * WTM) * q.N + (int64_t)nt * BN + wn * WTN;
   char* sbuf = smem + wave * (WTM * St::LD);
   const int lrow = lane & 31, lq = 4 * (lane >> 5);
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int r = 32 * i + lrow;
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        const int c = 32 * j + 8 * qd + lq;
-        float v[4] = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
-        if (p.accumulate) {
-          float old[4];
-          unpack4(*reinterpret_cast<const u32x2_t*>(C + (int64_t)r * q.N + c), old);
-#pragma unroll
-          for (int t2 = 0; t2 < 4; ++t2) v[t2] += old[t2];
-        }
-        St::put(sbuf, r, c, pack4(v[0], v[1], v[2], v[3]));
-      }
-  }
+      for (int qd = 0; qd < 4; ++qd)
+        St::put(sbuf, 32 * i + lrow, 32 * j + 8 * qd + lq,
+                pack4(acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]));
   wave_lds_fence();
-  St::template flush<WTM>(sbuf, C, q.N, WTM);
+  if (p.accumulate) St::template flush<WTM, true>(sbuf, C, q.N, WTM);
+  else St::template flush<WTM, false>(sbuf, C, q.N, WTM);
 }
 
 inline int round_up_xcd(int64_t n) { return (int)(pk_ceil_div(n, NXCD) * NXCD); }
@@ -634,15 +702,37 @@ int simt_ragged_k(const void* A, int64_t lda, const int32_t* a_map, const void* 
   return pk_simt::launch<T, T, T>(p, s);
 }
 
-// Tile configurations: BM, BN, waves along M, waves along N, LDS stages.
-#define PK_RM_BIG 128, 256, 2, 4, 3     /* 8 waves, 64x64 wave tiles, 144 KB ring */
-#define PK_RM_SMALL 128, 128, 2, 2, 3   /* 4 waves, 64x64 wave tiles,  96 KB ring */
-#define PK_WG_BIG 256, 256, 2, 2, 2     /* 4 waves, 128x128 wave tiles, 128 KB ring */
-#define PK_WG_BIG_THREADS 256
+// Tile configurations: BM, BN, waves along M, waves along N, LDS stages.  Measured on MI355X
+// with random data and multinomial / Zipf row counts over {128,256}x{128,256} tiles, 4/8/16
+// waves and 2/3 stages: 128x256 with 8 waves (64x64 wave tiles, 3-stage 144 KB ring) is fastest
+// for the ragged-M kernels, 256x256 with 8 waves (128x64 wave tiles) for the weight gradient.
+#ifndef PK_RM_CFG
+#define PK_RM_CFG 128, 256, 2, 4, 3
+#define PK_RM_BN 256
+#endif
+#ifndef PK_WG_BIG
+#define PK_WG_BIG 256, 256, 2, 4, 2     /* 8 waves, 128x64 wave tiles, 128 KB ring */
+#define PK_WG_BIG_THREADS 512
+#endif
 #define PK_WG_SMALL 128, 128, 2, 2, 3
 #define PK_WG_SMALL_THREADS 256
 
+#define PK_RM_ALT 128, 128, 2, 2, 3      /* output widths that are a multiple of 128 but not of 256 */
 bool mfma_shape_ok(int64_t H, int64_t I) { return H % 128 == 0 && I % 128 == 0; }
+
+// Pick the tile width by the output width N of the GEMM (for the gate/up kernel a tile holds
+// BN/2 gate and BN/2 up columns).
+template <bool B_KC, int EPI>
+int launch_rm(mf::RaggedMParams& p, int64_t A, int64_t N, int kernel_id, hipStream_t s) {
+  const int64_t per_tile_big = (EPI == mf::EPI_SWIGLU) ? PK_RM_BN / 2 : PK_RM_BN;
+  if (N % per_tile_big == 0) {
+    p.n_tiles = (int32_t)(N / per_tile_big);
+    return mf::launch_ragged_m<PK_RM_CFG, B_KC, EPI>(p, A, kernel_id, s);
+  }
+  const int64_t per_tile_alt = (EPI == mf::EPI_SWIGLU) ? 64 : 128;
+  p.n_tiles = (int32_t)(N / per_tile_alt);
+  return mf::launch_ragged_m<PK_RM_ALT, B_KC, EPI>(p, A, kernel_id, s);
+}
 
 bool all_aligned16(std::initializer_list<const void*> ptrs) {
   for (const void* p : ptrs)
@@ -729,8 +819,7 @@ int pk_grouped_swiglu_fwd(const void* x_rows, const int32_t* row_map, int64_t ro
   p.B0 = (const bf16_t*)w1; p.B1 = (const bf16_t*)w3; p.ldb = H; p.strideB = I * H;
   p.starts = starts; p.E = (int32_t)E; p.Kseg = (int32_t)H; p.nseg = 1;
   p.O0 = (bf16_t*)g; p.O1 = (bf16_t*)u; p.O2 = (bf16_t*)h; p.ldc = I;
-  p.n_tiles = (int32_t)(I / 128);   // a 256-row weight tile = 128 gate + 128 up columns
-  rc = mf::launch_ragged_m<PK_RM_BIG, true, mf::EPI_SWIGLU>(p, A, pk_timing::K_SWIGLU_GATE_UP, s);
+  rc = launch_rm<true, mf::EPI_SWIGLU>(p, A, I, pk_timing::K_SWIGLU_GATE_UP, s);
   if (rc) return rc;
 
   mf::RaggedMParams q = {};
@@ -738,12 +827,7 @@ int pk_grouped_swiglu_fwd(const void* x_rows, const int32_t* row_map, int64_t ro
   q.B0 = (const bf16_t*)w2; q.B1 = nullptr; q.ldb = I; q.strideB = H * I;
   q.starts = starts; q.E = (int32_t)E; q.Kseg = (int32_t)I; q.nseg = 1;
   q.O0 = (bf16_t*)y; q.ldc = H;
-  if (H % 256 == 0) {
-    q.n_tiles = (int32_t)(H / 256);
-    return mf::launch_ragged_m<PK_RM_BIG, true, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DOWN, s);
-  }
-  q.n_tiles = (int32_t)(H / 128);
-  return mf::launch_ragged_m<PK_RM_SMALL, true, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DOWN, s);
+  return launch_rm<true, mf::EPI_PLAIN>(q, A, H, pk_timing::K_SWIGLU_DOWN, s);
 }
 
 int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, const void* w3,
@@ -768,13 +852,7 @@ int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, con
   p.starts = starts; p.E = (int32_t)E; p.Kseg = (int32_t)H; p.nseg = 1;
   p.Gin = (const bf16_t*)g; p.Uin = (const bf16_t*)u;
   p.O0 = (bf16_t*)d_g; p.O1 = (bf16_t*)d_u; p.ldc = I;
-  if (I % 256 == 0) {
-    p.n_tiles = (int32_t)(I / 256);
-    rc = mf::launch_ragged_m<PK_RM_BIG, false, mf::EPI_SWIGLU_BWD>(p, A, pk_timing::K_SWIGLU_DGRAD_DH, s);
-  } else {
-    p.n_tiles = (int32_t)(I / 128);
-    rc = mf::launch_ragged_m<PK_RM_SMALL, false, mf::EPI_SWIGLU_BWD>(p, A, pk_timing::K_SWIGLU_DGRAD_DH, s);
-  }
+  rc = launch_rm<false, mf::EPI_SWIGLU_BWD>(p, A, I, pk_timing::K_SWIGLU_DGRAD_DH, s);
   if (rc) return rc;
 
   // d_x = [d_g | d_u] . [w1[e] ; w3[e]]
@@ -783,12 +861,7 @@ int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, con
   q.B0 = (const bf16_t*)w1; q.B1 = (const bf16_t*)w3; q.ldb = H; q.strideB = I * H;
   q.starts = starts; q.E = (int32_t)E; q.Kseg = (int32_t)I; q.nseg = 2;
   q.O0 = (bf16_t*)d_x_sorted; q.ldc = H;
-  if (H % 256 == 0) {
-    q.n_tiles = (int32_t)(H / 256);
-    return mf::launch_ragged_m<PK_RM_BIG, false, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DGRAD_DX, s);
-  }
-  q.n_tiles = (int32_t)(H / 128);
-  return mf::launch_ragged_m<PK_RM_SMALL, false, mf::EPI_PLAIN>(q, A, pk_timing::K_SWIGLU_DGRAD_DX, s);
+  return launch_rm<false, mf::EPI_PLAIN>(q, A, H, pk_timing::K_SWIGLU_DGRAD_DX, s);
 }
 
 int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, const void* d_u,
@@ -833,15 +906,18 @@ int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, con
   if (n == 0) return PK_OK;
   p.starts = starts; p.E = (int32_t)E; p.map_div = (int32_t)row_map_div;
   p.accumulate = accumulate ? 1 : 0;
+#ifdef PK_GEMM_DEBUG
+  { const char* d = getenv("PK_GEMM_DEBUG_MODE"); p.debug = d ? atoi(d) : 0; }
+#endif
   const bool big = (H % 256 == 0) && (I % 256 == 0);
   const int tile = big ? 256 : 128;
   p.tiles_per_expert = (int32_t)((H / tile) * (I / tile));
-  const int64_t blocks = (int64_t)p.tiles_per_expert * E;
+  const int64_t blocks = (int64_t)p.tiles_per_expert * pk_ceil_div(E, mf::NXCD) * mf::NXCD;
   if (blocks > 0x7ffffff0ll) return PK_ERR_SHAPE;
   if (big)
-    PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_WGRAD, s, (mf::wgrad_kernel<PK_WG_BIG>), dim3(mf::round_up_xcd(blocks), n), dim3(PK_WG_BIG_THREADS), 0, s, p);
+    PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_WGRAD, s, (mf::wgrad_kernel<PK_WG_BIG>), dim3((unsigned)blocks, n), dim3(PK_WG_BIG_THREADS), 0, s, p);
   else
-    PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_WGRAD, s, (mf::wgrad_kernel<PK_WG_SMALL>), dim3(mf::round_up_xcd(blocks), n), dim3(PK_WG_SMALL_THREADS), 0, s, p);
+    PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_WGRAD, s, (mf::wgrad_kernel<PK_WG_SMALL>), dim3((unsigned)blocks, n), dim3(PK_WG_SMALL_THREADS), 0, s, p);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
 }
