@@ -33,6 +33,9 @@ def parse_args():
     ap.add_argument("--workload", choices=["cfg3", "cfg4"], default="cfg3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bucket", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB fp32 device copy (pack_kernel<float,float>) so that "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled to a known size")
     return ap.parse_args()
 
 
@@ -201,6 +204,15 @@ def main():
         sys.exit(1)
     _lib.load()
     cfg = CFG3 if args.workload == "cfg3" else CFG4
+    if args.copy_calibration:
+        from piper_amd import ops
+        n = 64 * 1024 * 1024
+        src = torch.ones(n, device="cuda:0")
+        dst = torch.zeros(n, device="cuda:0")
+        for _ in range(3):
+            ops.bucket_pack([src], [0], dst, accumulate=False)   # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
     elapsed, kernels = bench_region(cfg, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = cfg.tokens * args.steps / elapsed

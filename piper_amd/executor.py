@@ -113,6 +113,7 @@ class StageExecutor:
     pack_stream: torch.cuda.Stream | None = None
     loss_fn: Any = None
     _fwd: dict = field(default_factory=dict)
+    _inp_grads: dict = field(default_factory=dict)
 
     def __post_init__(self):
         self.params = self.params or ParamStorage(self.stages)
@@ -125,6 +126,7 @@ class StageExecutor:
         cs = self.compute_stream or torch.cuda.current_stream()
         ps = self.pack_stream or cs
         self._fwd.clear()
+        self._inp_grads.clear()
         losses = []
         pack_events: dict = {}
         self.params.clear_param_grads()
@@ -159,8 +161,16 @@ class StageExecutor:
                     self.compute.backward(task.ubid, task.mb, [loss], None, None, None,
                                           rec["inp_with_grad"], rec["out_with_grad"], cs)
                 else:
+                    # the downstream bucket's input grads become the grads of this bucket's detached
+                    # outputs (src/executors.py:826-842)
+                    prev = self._inp_grads.pop((ubids[pos + 1], task.mb))
+                    for d, g in zip(rec["detached_outs"], prev):
+                        if isinstance(d, torch.Tensor) and d.requires_grad and g is not None:
+                            d.grad = g
                     self.compute.backward(task.ubid, task.mb, rec["pre_detach_outs"], None, rec["pre_detach_outs"],
                                           rec["detached_outs"], rec["inp_with_grad"], rec["out_with_grad"], cs)
+                self._inp_grads[(task.ubid, task.mb)] = [
+                    t.grad if (isinstance(t, torch.Tensor) and t.requires_grad) else None for t in rec["fwd_inputs"]]
                 # gradient pack on the second stream, ordered after this backward
                 if ps is not cs:
                     evt = torch.cuda.Event()
