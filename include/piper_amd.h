@@ -165,6 +165,15 @@ PK_API int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* 
                             void* d_u, void* d_x_sorted, int64_t A, int64_t H, int64_t I,
                             int64_t E, int dtype, pk_stream_t stream);
 
+/* The two halves of pk_grouped_swiglu_dgrad as separate launches, so that a caller can start
+ * the weight gradient (which needs d_g, d_u but not d_x) as soon as the first half is queued. */
+PK_API int pk_grouped_swiglu_dgrad_dh(const void* d_y, const void* w2, const void* g, const void* u,
+                               const int32_t* starts, void* d_g, void* d_u, int64_t A, int64_t H,
+                               int64_t I, int64_t E, int dtype, pk_stream_t stream);
+PK_API int pk_grouped_swiglu_dgrad_dx(const void* d_g, const void* d_u, const void* w1, const void* w3,
+                               const int32_t* starts, void* d_x_sorted, int64_t A, int64_t H,
+                               int64_t I, int64_t E, int dtype, pk_stream_t stream);
+
 /* Weight gradient (Piper's BWD_W task, src/executors.py:413-476).
  *   d_w2[e] (+)= d_y[rows_e]^T . h[rows_e]          [H,I]
  *   d_w1[e] (+)= d_g[rows_e]^T . x[rows_e]          [I,H]

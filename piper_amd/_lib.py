@@ -43,6 +43,8 @@ SIGNATURES = {
                                        _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
     "pk_grouped_swiglu_dgrad": (_c_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p,
                                          _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
+    "pk_grouped_swiglu_dgrad_dh": (_c_int, [_p, _p, _p, _p, _p, _p, _p, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
+    "pk_grouped_swiglu_dgrad_dx": (_c_int, [_p, _p, _p, _p, _p, _p, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
     "pk_grouped_swiglu_wgrad": (_c_int, [_p, _p, _p, _p, _p, _p, _c_i64, _p, _p, _p, _p, _c_int,
                                          _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
     "pk_bucket_plan": (_c_i64, [_p, _c_i64, _c_i64, _c_i64, _p]),

@@ -13,7 +13,6 @@ namespace {
 // ===================================================================== bf16 MFMA path
 namespace mf {
 
-constexpr int BK = 64, THREADS = 256;
 constexpr int NXCD = 8;
 
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_SWIGLU_BWD = 2 };
@@ -56,12 +55,12 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// LDS tile layouts.  Both are ROWS*128 bytes; 16-byte chunks are XOR-swizzled so that the
-// fragment reads below touch every bank once.
+// LDS tile layouts (BK = 64 or 32 deep).  16-byte chunks are XOR-swizzled so that the fragment
+// reads below touch every bank once.
 //
-// KC tile: [ROWS rows of the M or N index][64 k], k contiguous (128 B per row, 8 chunks).
-//          chunk c of row r sits at position c ^ ((r >> 1) & 7).
-// MN tile: [64 k][COLS of the M or N index], the M/N index contiguous (COLS/8 chunks per row).
+// KC tile: [ROWS rows of the M or N index][BK k], k contiguous (2*BK bytes per row, BK/8 chunks).
+//          chunk c of row r sits at position c ^ swz(r): (r >> 1) & 7 for BK 64, (r >> 2) & 3 for BK 32.
+// MN tile: [BK k][COLS of the M or N index], the M/N index contiguous (COLS/8 chunks per row).
 //          chunk c of row k sits at position c ^ ((k & 3) << 2).
 //
 // A wave-level dma16 fills 64 consecutive 16-byte slots; which global chunk a lane fetches is
@@ -69,9 +68,14 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 
 // Global element offset (within the operand) of the chunk that lane `lane` of load `G`
 // (G-th group of 64 slots of the tile) must fetch, for a KC tile: returns row and k offset.
+template <int BK>
+__device__ __forceinline__ int kc_swz(int row) { return BK == 64 ? ((row >> 1) & 7) : ((row >> 2) & 3); }
+template <int BK>
 __device__ __forceinline__ void kc_slot(int G, int lane, int& row, int& kofs) {
-  row = G * 8 + (lane >> 3);
-  kofs = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+  constexpr int CPR = BK / 8;
+  const int slot = G * 64 + lane;
+  row = slot / CPR;
+  kofs = ((slot % CPR) ^ kc_swz<BK>(row)) * 8;
 }
 template <int COLS>
 __device__ __forceinline__ void mn_slot(int G, int lane, int& krow, int& cofs) {
@@ -82,10 +86,11 @@ __device__ __forceinline__ void mn_slot(int G, int lane, int& krow, int& cofs) {
 }
 
 // MFMA operand fragment (8 bf16 per lane: row lane%32, k = 16*ks + 8*(lane/32) + 0..7).
+template <int BK>
 __device__ __forceinline__ bf16x8_t frag_kc(const char* tile, int row0, int ks, int lane) {
   const int r = row0 + (lane & 31);
   const int c = 2 * ks + (lane >> 5);
-  return *reinterpret_cast<const bf16x8_t*>(tile + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
+  return *reinterpret_cast<const bf16x8_t*>(tile + r * (2 * BK) + ((c ^ kc_swz<BK>(r)) << 4));
 }
 // Same fragment out of an MN tile through the transposing LDS read: within 16 lanes, lane i
 // points at 4 consecutive columns of k-row i/4 and receives 4 consecutive k of column i.
@@ -109,15 +114,15 @@ struct Frags {
   bf16x8_t a[TM];
   bf16x8_t b[TN];
 };
-template <int TM, int TN, bool A_KC, bool B_KC, int ACOLS, int BCOLS>
+template <int BK, int TM, int TN, bool A_KC, bool B_KC, int ACOLS, int BCOLS>
 __device__ __forceinline__ void load_frags(Frags<TM, TN>& f, const char* At, const char* Bt,
                                            int wrow0, int wcol0, int ks, int lane) {
 #pragma unroll
   for (int i = 0; i < TM; ++i)
-    f.a[i] = A_KC ? frag_kc(At, wrow0 + 32 * i, ks, lane) : frag_mn<ACOLS>(At, wrow0 + 32 * i, ks, lane);
+    f.a[i] = A_KC ? frag_kc<BK>(At, wrow0 + 32 * i, ks, lane) : frag_mn<ACOLS>(At, wrow0 + 32 * i, ks, lane);
 #pragma unroll
   for (int j = 0; j < TN; ++j)
-    f.b[j] = B_KC ? frag_kc(Bt, wcol0 + 32 * j, ks, lane) : frag_mn<BCOLS>(Bt, wcol0 + 32 * j, ks, lane);
+    f.b[j] = B_KC ? frag_kc<BK>(Bt, wcol0 + 32 * j, ks, lane) : frag_mn<BCOLS>(Bt, wcol0 + 32 * j, ks, lane);
 }
 
 // One 64-deep k-tile of MFMAs, software pipelined: the fragments of k-step s+1 are requested
@@ -127,7 +132,7 @@ __device__ __forceinline__ void load_frags(Frags<TM, TN>& f, const char* At, con
 // The operands are passed swapped (B first) so that each lane's accumulator holds 4
 // CONSECUTIVE output columns of ONE output row:
 //   acc[i][j][v] = C[row = 32*i + lane%32][col = 32*j + 8*(v/4) + 4*(lane/32) + v%4]
-template <int TM, int TN, bool A_KC, bool B_KC, int ACOLS, int BCOLS, bool LEAN>
+template <int BK, int TM, int TN, bool A_KC, bool B_KC, int ACOLS, int BCOLS, bool LEAN>
 __device__ __forceinline__ void mma_tile(const char* At, const char* Bt, int wrow0, int wcol0,
                                          floatx16_t (&acc)[TM][TN]) {
   const int lane = threadIdx.x & 63;
@@ -136,16 +141,16 @@ __device__ __forceinline__ void mma_tile(const char* At, const char* Bt, int wro
     bf16x8_t a[TM], b[2][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-      a[i] = A_KC ? frag_kc(At, wrow0 + 32 * i, 0, lane) : frag_mn<ACOLS>(At, wrow0 + 32 * i, 0, lane);
+      a[i] = A_KC ? frag_kc<BK>(At, wrow0 + 32 * i, 0, lane) : frag_mn<ACOLS>(At, wrow0 + 32 * i, 0, lane);
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-      b[0][j] = B_KC ? frag_kc(Bt, wcol0 + 32 * j, 0, lane) : frag_mn<BCOLS>(Bt, wcol0 + 32 * j, 0, lane);
+      b[0][j] = B_KC ? frag_kc<BK>(Bt, wcol0 + 32 * j, 0, lane) : frag_mn<BCOLS>(Bt, wcol0 + 32 * j, 0, lane);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + 1 < KS) {
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          b[(ks + 1) & 1][j] = B_KC ? frag_kc(Bt, wcol0 + 32 * j, ks + 1, lane)
+          b[(ks + 1) & 1][j] = B_KC ? frag_kc<BK>(Bt, wcol0 + 32 * j, ks + 1, lane)
                                     : frag_mn<BCOLS>(Bt, wcol0 + 32 * j, ks + 1, lane);
       }
 #pragma unroll
@@ -154,21 +159,26 @@ __device__ __forceinline__ void mma_tile(const char* At, const char* Bt, int wro
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[ks & 1][j], a[i], acc[i][j], 0, 0, 0);
         if (ks + 1 < KS)
-          a[i] = A_KC ? frag_kc(At, wrow0 + 32 * i, ks + 1, lane) : frag_mn<ACOLS>(At, wrow0 + 32 * i, ks + 1, lane);
+          a[i] = A_KC ? frag_kc<BK>(At, wrow0 + 32 * i, ks + 1, lane) : frag_mn<ACOLS>(At, wrow0 + 32 * i, ks + 1, lane);
       }
     }
   } else {
     Frags<TM, TN> f[2];
-    load_frags<TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[0], At, Bt, wrow0, wcol0, 0, lane);
+    load_frags<BK, TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[0], At, Bt, wrow0, wcol0, 0, lane);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + 1 < KS)
-        load_frags<TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[(ks + 1) & 1], At, Bt, wrow0, wcol0, ks + 1, lane);
+        load_frags<BK, TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[(ks + 1) & 1], At, Bt, wrow0, wcol0, ks + 1, lane);
+      // keep the LDS reads of the next k-step ahead of this k-step's MFMAs: without the fence
+      // the scheduler sinks them behind the MFMAs to reuse the fragment registers, which
+      // exposes the LDS latency once per k-step
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[ks & 1].b[j], f[ks & 1].a[i], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 }
@@ -298,13 +308,13 @@ struct RaggedMParams {
 // Block tile BM x BN, WMW x WNW waves, NS-stage LDS ring filled by direct-to-LDS loads.
 // EPI_SWIGLU: the BN tile rows are [32 gate | 32 up | 32 gate | 32 up ...] of BN/2 output
 // columns, so that a lane holds the gate and the up value of the same element.
-template <int BM, int BN, int WMW, int WNW, int NS, bool B_KC, int EPI>
-__global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMParams p) {
+template <int BM, int BN, int BK, int WMW, int WNW, int NS, int OCC, bool B_KC, int EPI>
+__global__ __launch_bounds__(64 * WMW * WNW, OCC * WMW * WNW / 4) void ragged_m_kernel(const RaggedMParams p) {
   constexpr int NTHREADS = 64 * WMW * WNW;
   constexpr int WTM = BM / WMW, WTN = BN / WNW;          // wave tile
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr int A_BYTES = BM * 128, STAGE = (BM + BN) * 128;
-  constexpr int LA = BM * 8 / NTHREADS, LB = BN * 8 / NTHREADS;   // dma16 per thread per tile
+  constexpr int A_BYTES = BM * BK * 2, STAGE = (BM + BN) * BK * 2;
+  constexpr int LA = A_BYTES / (NTHREADS * 16), LB = (STAGE - A_BYTES) / (NTHREADS * 16);   // dma16 per thread per tile
   static_assert(LA >= 1 && LB >= 1 && TM >= 1 && TN >= 1, "tile too small for the wave grid");
   static_assert(EPI != EPI_SWIGLU || (WTN % 64 == 0), "gate/up pairs must stay inside a wave");
   // output columns a wave writes per output tensor, and its staging buffer
@@ -328,7 +338,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
 #pragma unroll
   for (int i = 0; i < LA; ++i) {
     int r, kofs;
-    kc_slot(wave * LA + i, lane, r, kofs);
+    kc_slot<BK>(wave * LA + i, lane, r, kofs);
     r = r < rows ? r : rows - 1;     // clamp: rows past the expert's range are never stored
     int64_t src = row0 + r;
     if (p.row_map) src = p.row_map[src] / p.map_div;
@@ -342,7 +352,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     b_mat[i] = 0;
     if (B_KC) {
       int r, kofs;
-      kc_slot(wave * LB + i, lane, r, kofs);
+      kc_slot<BK>(wave * LB + i, lane, r, kofs);
       int n;
       if (EPI == EPI_SWIGLU) {
         b_mat[i] = (r >> 5) & 1;
@@ -403,7 +413,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     if (!(p.debug & 1))
 #endif
     if (wave_has_rows)
-      mma_tile<TM, TN, true, B_KC, BM, BN, false>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
+      mma_tile<BK, TM, TN, true, B_KC, BM, BN, false>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
     cur = cur + 1 == NS ? 0 : cur + 1;
     nxt = nxt + 1 == NS ? 0 : nxt + 1;
   }
@@ -502,13 +512,13 @@ struct WgradParams {
 #endif
 };
 
-template <int BM, int BN, int WMW, int WNW, int NS>
+template <int BM, int BN, int BK, int WMW, int WNW, int NS>
 __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams p) {
   constexpr int NTHREADS = 64 * WMW * WNW;
   constexpr int WTM = BM / WMW, WTN = BN / WNW;
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr int A_BYTES = BM * 128, STAGE = (BM + BN) * 128;
-  constexpr int LA = BM * 8 / NTHREADS, LB = BN * 8 / NTHREADS;
+  constexpr int A_BYTES = BM * BK * 2, STAGE = (BM + BN) * BK * 2;
+  constexpr int LA = A_BYTES / (NTHREADS * 16), LB = (STAGE - A_BYTES) / (NTHREADS * 16);
   using St = Stage<WTN>;
   constexpr int STAGING = WTM * St::LD * (WMW * WNW);
   constexpr int SMEM = STAGING > NS * STAGE ? STAGING : NS * STAGE;
@@ -606,7 +616,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
 #ifdef PK_GEMM_DEBUG
     if (!(p.debug & 1))
 #endif
-    mma_tile<TM, TN, false, false, BM, BN, (TM * TN >= 16)>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
+    mma_tile<BK, TM, TN, false, false, BM, BN, (TM * TN >= 16)>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
     cur = cur + 1 == NS ? 0 : cur + 1;
     nxt = nxt + 1 == NS ? 0 : nxt + 1;
   }
@@ -633,14 +643,14 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
 
 inline int round_up_xcd(int64_t n) { return (int)(pk_ceil_div(n, NXCD) * NXCD); }
 
-template <int BM, int BN, int WMW, int WNW, int NS, bool B_KC, int EPI>
+template <int BM, int BN, int BK, int WMW, int WNW, int NS, int OCC, bool B_KC, int EPI>
 int launch_ragged_m(RaggedMParams p, int64_t A_rows, int kernel_id, hipStream_t s) {
 #ifdef PK_GEMM_DEBUG
   { const char* d = getenv("PK_GEMM_DEBUG_MODE"); p.debug = d ? atoi(d) : 0; }
 #endif
   const int64_t max_units = (pk_ceil_div(A_rows, BM) + p.E) * p.n_tiles;
   if (max_units > 0x7ffffff0ll) return PK_ERR_SHAPE;
-  PK_LAUNCH_NOCHECK(kernel_id, s, (ragged_m_kernel<BM, BN, WMW, WNW, NS, B_KC, EPI>),
+  PK_LAUNCH_NOCHECK(kernel_id, s, (ragged_m_kernel<BM, BN, BK, WMW, WNW, NS, OCC, B_KC, EPI>),
                     dim3(round_up_xcd(max_units)), dim3(64 * WMW * WNW), 0, s, p);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
@@ -706,18 +716,19 @@ int simt_ragged_k(const void* A, int64_t lda, const int32_t* a_map, const void* 
 // with random data and multinomial / Zipf row counts over {128,256}x{128,256} tiles, 4/8/16
 // waves and 2/3 stages: 128x256 with 8 waves (64x64 wave tiles, 3-stage 144 KB ring) is fastest
 // for the ragged-M kernels, 256x256 with 8 waves (128x64 wave tiles) for the weight gradient.
+// (BM, BN, BK, waves M, waves N, stages, workgroups per CU)
 #ifndef PK_RM_CFG
-#define PK_RM_CFG 128, 256, 2, 4, 3
+#define PK_RM_CFG 128, 256, 64, 2, 4, 3, 1
 #define PK_RM_BN 256
 #endif
 #ifndef PK_WG_BIG
-#define PK_WG_BIG 256, 256, 2, 4, 2     /* 8 waves, 128x64 wave tiles, 128 KB ring */
+#define PK_WG_BIG 256, 256, 64, 2, 4, 2     /* 8 waves, 128x64 wave tiles, 128 KB ring */
 #define PK_WG_BIG_THREADS 512
 #endif
-#define PK_WG_SMALL 128, 128, 2, 2, 3
+#define PK_WG_SMALL 128, 128, 64, 2, 2, 3
 #define PK_WG_SMALL_THREADS 256
 
-#define PK_RM_ALT 128, 128, 2, 2, 3      /* output widths that are a multiple of 128 but not of 256 */
+#define PK_RM_ALT 128, 128, 64, 2, 2, 3, 1      /* output widths that are a multiple of 128 but not of 256 */
 bool mfma_shape_ok(int64_t H, int64_t I) { return H % 128 == 0 && I % 128 == 0; }
 
 // Pick the tile width by the output width N of the GEMM (for the gate/up kernel a tile holds
@@ -760,23 +771,6 @@ int fwd_simt(const void* x, const int32_t* row_map, int64_t div, const void* w1,
                      (const T*)g, (const T*)u, (T*)h, n);
   PK_RETURN_IF_LAUNCH_FAILED();
   return simt_ragged_m<T>(h, I, nullptr, 1, w2, 1, I, H * I, y, H, starts, A, H, I, E, 0, s);
-}
-
-template <typename T>
-int dgrad_simt(const void* dy, const void* w1, const void* w2, const void* w3, const void* g,
-               const void* u, const int32_t* starts, void* dg, void* du, void* dx, int64_t A,
-               int64_t H, int64_t I, int64_t E, hipStream_t s) {
-  // d_h = d_y . w2[e]  (w2[e] is [H, I]: B(k=h, n=i) = w2[h*I + i]); staged in d_u's buffer
-  int rc = simt_ragged_m<T>(dy, H, nullptr, 1, w2, I, 1, H * I, du, I, starts, A, I, H, E, 0, s);
-  if (rc) return rc;
-  const int64_t n = A * I;
-  PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_ELEMENTWISE, s, (swiglu_bwd_kernel<T>), dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
-                     (const T*)du, (const T*)g, (const T*)u, (T*)dg, (T*)du, n);
-  PK_RETURN_IF_LAUNCH_FAILED();
-  // d_x = d_g . w1[e] + d_u . w3[e]   (w[e] is [I, H]: B(k=i, n=h) = w[i*H + h])
-  rc = simt_ragged_m<T>(dg, I, nullptr, 1, w1, H, 1, I * H, dx, H, starts, A, H, I, E, 0, s);
-  if (rc) return rc;
-  return simt_ragged_m<T>(du, I, nullptr, 1, w3, H, 1, I * H, dx, H, starts, A, H, I, E, 1, s);
 }
 
 template <typename T>
@@ -830,31 +824,61 @@ int pk_grouped_swiglu_fwd(const void* x_rows, const int32_t* row_map, int64_t ro
   return launch_rm<true, mf::EPI_PLAIN>(q, A, H, pk_timing::K_SWIGLU_DOWN, s);
 }
 
-int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, const void* w3,
-                            const void* g, const void* u, const int32_t* starts, void* d_g,
-                            void* d_u, void* d_x_sorted, int64_t A, int64_t H, int64_t I,
-                            int64_t E, int dtype, pk_stream_t stream) {
+int pk_grouped_swiglu_dgrad_dh(const void* d_y, const void* w2, const void* g, const void* u,
+                               const int32_t* starts, void* d_g, void* d_u, int64_t A, int64_t H,
+                               int64_t I, int64_t E, int dtype, pk_stream_t stream) {
   int rc = check_common(A, H, I, E, dtype);
   if (rc) return rc;
   if (A == 0) return PK_OK;
-  if (!d_y || !w1 || !w2 || !w3 || !g || !u || !starts || !d_g || !d_u || !d_x_sorted)
-    return PK_ERR_ARG;
+  if (!d_y || !w2 || !g || !u || !starts || !d_g || !d_u) return PK_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == PK_F32)
-    return dgrad_simt<float>(d_y, w1, w2, w3, g, u, starts, d_g, d_u, d_x_sorted, A, H, I, E, s);
-  if (!mfma_shape_ok(H, I) || !all_aligned16({d_y, w1, w2, w3, g, u, d_g, d_u, d_x_sorted}))
-    return dgrad_simt<bf16_t>(d_y, w1, w2, w3, g, u, starts, d_g, d_u, d_x_sorted, A, H, I, E, s);
-
-  // d_h = d_y . w2[e]  ->  (d_g, d_u) in the epilogue
+  const bool simt = dtype == PK_F32 || !mfma_shape_ok(H, I) || !all_aligned16({d_y, w2, g, u, d_g, d_u});
+  if (simt) {
+    // d_h = d_y . w2[e]  (w2[e] is [H, I]: B(k=h, n=i) = w2[h*I + i]); staged in d_u's buffer
+    const int64_t n = A * I;
+    if (dtype == PK_F32) {
+      rc = simt_ragged_m<float>(d_y, H, nullptr, 1, w2, I, 1, H * I, d_u, I, starts, A, I, H, E, 0, s);
+      if (rc) return rc;
+      PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_ELEMENTWISE, s, (swiglu_bwd_kernel<float>), dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
+                        (const float*)d_u, (const float*)g, (const float*)u, (float*)d_g, (float*)d_u, n);
+    } else {
+      rc = simt_ragged_m<bf16_t>(d_y, H, nullptr, 1, w2, I, 1, H * I, d_u, I, starts, A, I, H, E, 0, s);
+      if (rc) return rc;
+      PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_ELEMENTWISE, s, (swiglu_bwd_kernel<bf16_t>), dim3((unsigned)pk_ceil_div(n, 256)), dim3(256), 0, s,
+                        (const bf16_t*)d_u, (const bf16_t*)g, (const bf16_t*)u, (bf16_t*)d_g, (bf16_t*)d_u, n);
+    }
+    PK_RETURN_IF_LAUNCH_FAILED();
+    return PK_OK;
+  }
   mf::RaggedMParams p = {};
   p.A0 = (const bf16_t*)d_y; p.lda = H;
   p.B0 = (const bf16_t*)w2; p.ldb = I; p.strideB = H * I;
   p.starts = starts; p.E = (int32_t)E; p.Kseg = (int32_t)H; p.nseg = 1;
   p.Gin = (const bf16_t*)g; p.Uin = (const bf16_t*)u;
   p.O0 = (bf16_t*)d_g; p.O1 = (bf16_t*)d_u; p.ldc = I;
-  rc = launch_rm<false, mf::EPI_SWIGLU_BWD>(p, A, I, pk_timing::K_SWIGLU_DGRAD_DH, s);
-  if (rc) return rc;
+  return launch_rm<false, mf::EPI_SWIGLU_BWD>(p, A, I, pk_timing::K_SWIGLU_DGRAD_DH, s);
+}
 
+int pk_grouped_swiglu_dgrad_dx(const void* d_g, const void* d_u, const void* w1, const void* w3,
+                               const int32_t* starts, void* d_x_sorted, int64_t A, int64_t H,
+                               int64_t I, int64_t E, int dtype, pk_stream_t stream) {
+  int rc = check_common(A, H, I, E, dtype);
+  if (rc) return rc;
+  if (A == 0) return PK_OK;
+  if (!d_g || !d_u || !w1 || !w3 || !starts || !d_x_sorted) return PK_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const bool simt = dtype == PK_F32 || !mfma_shape_ok(H, I) || !all_aligned16({d_g, d_u, w1, w3, d_x_sorted});
+  if (simt) {
+    // d_x = d_g . w1[e] + d_u . w3[e]   (w[e] is [I, H]: B(k=i, n=h) = w[i*H + h])
+    if (dtype == PK_F32) {
+      rc = simt_ragged_m<float>(d_g, I, nullptr, 1, w1, H, 1, I * H, d_x_sorted, H, starts, A, H, I, E, 0, s);
+      if (rc) return rc;
+      return simt_ragged_m<float>(d_u, I, nullptr, 1, w3, H, 1, I * H, d_x_sorted, H, starts, A, H, I, E, 1, s);
+    }
+    rc = simt_ragged_m<bf16_t>(d_g, I, nullptr, 1, w1, H, 1, I * H, d_x_sorted, H, starts, A, H, I, E, 0, s);
+    if (rc) return rc;
+    return simt_ragged_m<bf16_t>(d_u, I, nullptr, 1, w3, H, 1, I * H, d_x_sorted, H, starts, A, H, I, E, 1, s);
+  }
   // d_x = [d_g | d_u] . [w1[e] ; w3[e]]
   mf::RaggedMParams q = {};
   q.A0 = (const bf16_t*)d_g; q.A1 = (const bf16_t*)d_u; q.lda = I;
@@ -862,6 +886,15 @@ int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, con
   q.starts = starts; q.E = (int32_t)E; q.Kseg = (int32_t)I; q.nseg = 2;
   q.O0 = (bf16_t*)d_x_sorted; q.ldc = H;
   return launch_rm<false, mf::EPI_PLAIN>(q, A, H, pk_timing::K_SWIGLU_DGRAD_DX, s);
+}
+
+int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, const void* w3,
+                            const void* g, const void* u, const int32_t* starts, void* d_g,
+                            void* d_u, void* d_x_sorted, int64_t A, int64_t H, int64_t I,
+                            int64_t E, int dtype, pk_stream_t stream) {
+  int rc = pk_grouped_swiglu_dgrad_dh(d_y, w2, g, u, starts, d_g, d_u, A, H, I, E, dtype, stream);
+  if (rc) return rc;
+  return pk_grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts, d_x_sorted, A, H, I, E, dtype, stream);
 }
 
 int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, const void* d_u,

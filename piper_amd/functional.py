@@ -169,6 +169,27 @@ def combine(gathered_output, token_indices_experts_sorted, top_scores):
 
 
 # --------------------------------------------------------------------------- fused region
+# Measured on MI355X: running the weight gradient next to the input gradient gains ~1.5 % (both
+# kernels are throughput-bound), so it is opt-in; per-kernel timings are only meaningful with it off.
+_OVERLAP_WGRAD = False
+_SIDE_STREAMS: dict = {}
+
+
+def set_overlap_wgrad(on: bool) -> None:
+    """Run the weight-gradient kernel on a second stream, concurrently with the input gradient."""
+    global _OVERLAP_WGRAD
+    _OVERLAP_WGRAD = bool(on)
+
+
+def _side_stream(device) -> torch.cuda.Stream:
+    """One extra default-priority stream per device for the weight-gradient kernel."""
+    key = torch.device(device).index or 0
+    st = _SIDE_STREAMS.get(key)
+    if st is None:
+        st = torch.cuda.Stream(device=device)
+        _SIDE_STREAMS[key] = st
+    return st
+
 
 
 class _ExpertRegionFn(torch.autograd.Function):
@@ -193,15 +214,31 @@ class _ExpertRegionFn(torch.autograd.Function):
         E = w1.shape[0]
         need = ctx.needs_input_grad
         d_y, d_scores = ops.combine_bwd(d_out, y, perm, top_scores)
-        d_xs, d_g, d_u = ops.grouped_swiglu_dgrad(d_y, w1, w2, w3, g, u, starts)
+        d_g, d_u = ops.grouped_swiglu_dgrad_dh(d_y, w2, g, u, starts)
+        # The weight gradient (Piper's BWD_W) depends only on d_y, h, d_g, d_u and x; it runs on a
+        # second stream next to the input gradient (BWD_I) so the two kernels fill each other's tails.
         d_w1 = d_w2 = d_w3 = None
+        cur = torch.cuda.current_stream(x.device)
+        side = _side_stream(x.device) if (need[3] or need[4] or need[5]) and _OVERLAP_WGRAD else None
         if need[3] or need[4] or need[5]:
-            d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k)
+            if side is not None:
+                side.wait_stream(cur)
+                with torch.cuda.stream(side):
+                    d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k)
+            else:
+                d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k)
+        d_xs = ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
         d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
         d_wg = torch.empty_like(w_gate) if need[1] else None
         d_b = torch.empty(E, dtype=torch.float32, device=x.device) if (has_bias and need[2]) else None
         d_x32 = ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=need[0], d_w_gate=d_wg, d_gate_bias=d_b)
         d_x = ops.permute_bwd(d_xs, inv_perm, top_k, addend_f32=d_x32) if need[0] else None
+        if side is not None:
+            cur.wait_stream(side)
+            for t in (d_y, d_g, d_u):        # allocated on the current stream, read on the side stream
+                t.record_stream(side)
+            for t in (d_w1, d_w2, d_w3):     # allocated on the side stream, consumed on the current one
+                t.record_stream(cur)
         return d_x, d_wg, d_b, d_w1, d_w2, d_w3, None, None, None
 
 

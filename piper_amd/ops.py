@@ -199,6 +199,29 @@ def grouped_swiglu_dgrad(d_y, w1, w2, w3, g, u, starts):
     return d_x, d_g, d_u
 
 
+def grouped_swiglu_dgrad_dh(d_y, w2, g, u, starts):
+    """First half of the input gradient: (d_g, d_u) [A,I] from d_y."""
+    require_gpu(d_y)
+    E, H, I = w2.shape
+    A = d_y.shape[0]
+    d_g = torch.empty_like(g)
+    d_u = torch.empty_like(u)
+    call("pk_grouped_swiglu_dgrad_dh", ptr(d_y.contiguous()), ptr(w2.contiguous()), ptr(g), ptr(u), ptr(starts),
+         ptr(d_g), ptr(d_u), A, H, I, E, dtype_code(d_y.dtype), current_stream(d_y.device))
+    return d_g, d_u
+
+
+def grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts):
+    """Second half of the input gradient: d_x_sorted [A,H] = d_g . w1 + d_u . w3."""
+    require_gpu(d_g)
+    E, I, H = w1.shape
+    A = d_g.shape[0]
+    d_x = torch.empty((A, H), dtype=d_g.dtype, device=d_g.device)
+    call("pk_grouped_swiglu_dgrad_dx", ptr(d_g), ptr(d_u), ptr(w1.contiguous()), ptr(w3.contiguous()), ptr(starts),
+         ptr(d_x), A, H, I, E, dtype_code(d_g.dtype), current_stream(d_g.device))
+    return d_x
+
+
 def grouped_swiglu_wgrad(d_y, h, d_g, d_u, x_rows, starts, E, *, row_map=None, row_map_div=1,
                          d_w1=None, d_w2=None, d_w3=None, accumulate=False):
     """Weight gradients.  Without d_w* buffers, fresh tensors are returned; with buffers and

@@ -132,6 +132,20 @@ def test_bf16_region_against_fp32_oracle(dev, cfg, fused):
         assert int((aux["counts"] == 0).sum()) > 0, "this case is meant to contain empty experts"
 
 
+def test_wgrad_on_side_stream_gives_identical_results(dev):
+    inp = make_expert_region_inputs(SMALL_BF16)
+    o1, g1 = _gpu_fwd_bwd(inp, SMALL_BF16, dev, fused=True)
+    F_.set_overlap_wgrad(True)
+    try:
+        o2, g2 = _gpu_fwd_bwd(inp, SMALL_BF16, dev, fused=True)
+        torch.cuda.synchronize()
+    finally:
+        F_.set_overlap_wgrad(False)
+    assert torch.equal(o1, o2)
+    for k in g1:
+        assert torch.equal(g1[k], g2[k]), k
+
+
 def test_fused_and_piecewise_paths_agree(dev):
     inp = make_expert_region_inputs(SMALL_BF16)
     o1, g1 = _gpu_fwd_bwd(inp, SMALL_BF16, dev, fused=True)
