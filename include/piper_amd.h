@@ -95,12 +95,14 @@ PK_API int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype,
  *   starts[E+1] i32  exclusive prefix sum, starts[E] = A        (qwen3_bmm_experts_patch.py:27)
  *   perm[A]     i32  sorted position -> flat slot  ("token_indices_experts_sorted")
  *   inv_perm[A] i32  flat slot -> sorted position
+ *   order[E]    i32  (may be NULL) experts by descending row count, ties by index; a
+ *                    scheduling hint for pk_grouped_swiglu_wgrad under skewed routing
  * Within an expert, slots stay in ascending order (= torch.argsort(stable=True)).
  * Replaces the reorderer call (qwen3.py:243-247).  Expert ids must lie in [0,E). */
 PK_API int64_t pk_sort_workspace_bytes(int64_t A, int64_t E);
 PK_API int pk_sort_by_expert(const int32_t* top_idx, int64_t A, int64_t E, int32_t* counts,
-                      int32_t* starts, int32_t* perm, int32_t* inv_perm, void* workspace,
-                      int64_t workspace_bytes, pk_stream_t stream);
+                      int32_t* starts, int32_t* perm, int32_t* inv_perm, int32_t* order,
+                      void* workspace, int64_t workspace_bytes, pk_stream_t stream);
 
 /* starts[E+1] (i32) from counts[E] given as int32 (counts_is_i64 == 0) or int64.
  * For callers that hand pk_grouped_swiglu_* a `num_tokens_per_expert` tensor
@@ -178,13 +180,16 @@ PK_API int pk_grouped_swiglu_dgrad_dx(const void* d_g, const void* d_u, const vo
  *   d_w2[e] (+)= d_y[rows_e]^T . h[rows_e]          [H,I]
  *   d_w1[e] (+)= d_g[rows_e]^T . x[rows_e]          [I,H]
  *   d_w3[e] (+)= d_u[rows_e]^T . x[rows_e]          [I,H]
- * x rows are addressed as in the forward (row_map / row_map_div).  accumulate != 0 adds
+ * x rows are addressed as in the forward (row_map / row_map_div).  expert_order (may be NULL)
+ * is the `order` output of pk_sort_by_expert; it only changes which compute units work on
+ * which expert, never the result.  accumulate != 0 adds
  * to the existing contents (gradient accumulation over microbatches,
  * src/executors.py:333-343); otherwise every element is overwritten, with zeros for
  * an expert that received no rows. */
 PK_API int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, const void* d_u,
                             const void* x_rows, const int32_t* row_map, int64_t row_map_div,
-                            const int32_t* starts, void* d_w1, void* d_w2, void* d_w3,
+                            const int32_t* starts, const int32_t* expert_order, void* d_w1,
+                            void* d_w2, void* d_w3,
                             int accumulate, int64_t A, int64_t H, int64_t I, int64_t E,
                             int dtype, pk_stream_t stream);
 

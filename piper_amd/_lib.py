@@ -33,7 +33,7 @@ SIGNATURES = {
     "pk_gate_bwd_workspace_bytes": (_c_i64, [_c_i64, _c_i64, _c_i64]),
     "pk_gate_logits_bwd": (_c_int, [_p, _p, _c_int, _p, _p, _p, _p, _c_int, _c_i64, _c_i64, _c_i64, _p, _c_i64, _p]),
     "pk_sort_workspace_bytes": (_c_i64, [_c_i64, _c_i64]),
-    "pk_sort_by_expert": (_c_int, [_p, _c_i64, _c_i64, _p, _p, _p, _p, _p, _c_i64, _p]),
+    "pk_sort_by_expert": (_c_int, [_p, _c_i64, _c_i64, _p, _p, _p, _p, _p, _p, _c_i64, _p]),
     "pk_counts_to_starts": (_c_int, [_p, _c_int, _c_i64, _p, _p]),
     "pk_permute_fwd": (_c_int, [_p, _c_int, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
     "pk_permute_bwd": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
@@ -45,7 +45,7 @@ SIGNATURES = {
                                          _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
     "pk_grouped_swiglu_dgrad_dh": (_c_int, [_p, _p, _p, _p, _p, _p, _p, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
     "pk_grouped_swiglu_dgrad_dx": (_c_int, [_p, _p, _p, _p, _p, _p, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
-    "pk_grouped_swiglu_wgrad": (_c_int, [_p, _p, _p, _p, _p, _p, _c_i64, _p, _p, _p, _p, _c_int,
+    "pk_grouped_swiglu_wgrad": (_c_int, [_p, _p, _p, _p, _p, _p, _c_i64, _p, _p, _p, _p, _p, _c_int,
                                          _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
     "pk_bucket_plan": (_c_i64, [_p, _c_i64, _c_i64, _c_i64, _p]),
     "pk_bucket_pack": (_c_int, [_p, _p, _p, _c_i64, _c_int, _p, _c_int, _c_int, _p]),

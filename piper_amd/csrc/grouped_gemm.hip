@@ -503,6 +503,7 @@ struct WgradProblem {
 struct WgradParams {
   WgradProblem prob[3];
   const int32_t* starts;
+  const int32_t* order;      // optional [E]: experts by descending row count
   int32_t E;
   int32_t map_div;
   int32_t accumulate;
@@ -525,15 +526,19 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
   __shared__ __attribute__((aligned(1024))) char smem[SMEM];
 
   const WgradProblem& q = p.prob[blockIdx.y];
-  // Experts are dealt round-robin to the 8 XCDs (workgroup b runs on XCD b % 8); the tiles of one
-  // expert stay on one XCD, back to back, so its rows are read from HBM once.
+  // Workgroup b runs on XCD b % 8.  All tiles of one expert stay on one XCD, back to back, so its
+  // rows are read from HBM once.  Experts are dealt to the XCDs in "snake" order (0..7, 7..0,
+  // 0..7, ...) of p.order, the experts sorted by descending row count (pk_sort_by_expert), which
+  // balances skewed routing; without an order they are dealt by index.
+  const const_i32_ptr starts = as_const(p.starts);
   const int xcd = blockIdx.x % NXCD, pos = blockIdx.x / NXCD;
-  const int e = xcd + NXCD * (pos / p.tiles_per_expert);
-  if (e >= p.E) return;
+  const int jq = pos / p.tiles_per_expert;                       // position in this XCD's queue
+  const int want = (jq & 1) ? jq * NXCD + (NXCD - 1 - xcd) : jq * NXCD + xcd;   // rank to serve
+  if (want >= p.E) return;
+  const int e = p.order ? as_const(p.order)[want] : want;
   const int t = pos % p.tiles_per_expert;
   const int n_tiles = q.N / BN;
   const int mt = t / n_tiles, nt = t % n_tiles;
-  const const_i32_ptr starts = as_const(p.starts);
   const int row_begin = starts[e], row_end = starts[e + 1];
   const int nkt = (row_end - row_begin + BK - 1) / BK;
 
@@ -899,7 +904,8 @@ int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, con
 
 int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, const void* d_u,
                             const void* x_rows, const int32_t* row_map, int64_t row_map_div,
-                            const int32_t* starts, void* d_w1, void* d_w2, void* d_w3,
+                            const int32_t* starts, const int32_t* expert_order, void* d_w1,
+                            void* d_w2, void* d_w3,
                             int accumulate, int64_t A, int64_t H, int64_t I, int64_t E,
                             int dtype, pk_stream_t stream) {
   int rc = check_common(A, H, I, E, dtype);
@@ -937,7 +943,7 @@ int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, con
     q.C = (bf16_t*)d_w3; q.M = (int32_t)I; q.N = (int32_t)H;
   }
   if (n == 0) return PK_OK;
-  p.starts = starts; p.E = (int32_t)E; p.map_div = (int32_t)row_map_div;
+  p.starts = starts; p.order = expert_order; p.E = (int32_t)E; p.map_div = (int32_t)row_map_div;
   p.accumulate = accumulate ? 1 : 0;
 #ifdef PK_GEMM_DEBUG
   { const char* d = getenv("PK_GEMM_DEBUG_MODE"); p.debug = d ? atoi(d) : 0; }

@@ -171,20 +171,29 @@ __global__ __launch_bounds__(64) void sort_hist_kernel(const int32_t* __restrict
 __global__ __launch_bounds__(1024) void sort_scan_kernel(int32_t* __restrict__ chunk_hist,
                                                          int nchunks, int E,
                                                          int32_t* __restrict__ counts,
-                                                         int32_t* __restrict__ starts) {
+                                                         int32_t* __restrict__ starts,
+                                                         int32_t* __restrict__ order) {
   __shared__ int32_t scan[PK_MAX_EXPERTS];
+  __shared__ int32_t cnts[PK_MAX_EXPERTS];
   const int e = threadIdx.x;
   int total = 0;
   if (e < E) {
-    for (int c = 0; c < nchunks; ++c) {
-      const int v = chunk_hist[(int64_t)c * E + e];
-      chunk_hist[(int64_t)c * E + e] = total;
-      total += v;
-    }
+    // pass 1 only reads (the loads pipeline), pass 2 rewrites each entry with its prefix
+    for (int c = 0; c < nchunks; ++c) total += chunk_hist[(int64_t)c * E + e];
     if (counts) counts[e] = total;
   }
   scan[e] = (e < E) ? total : 0;
+  cnts[e] = (e < E) ? total : -1;
   __syncthreads();
+  if (order && e < E) {
+    // experts by descending row count, ties by index: order[rank] = e
+    int rank = 0;
+    for (int o = 0; o < E; ++o) {
+      const int oc = cnts[o];
+      rank += (oc > total || (oc == total && o < e)) ? 1 : 0;
+    }
+    order[rank] = e;
+  }
   // Hillis-Steele inclusive scan over 1024 entries
   for (int off = 1; off < 1024; off <<= 1) {
     const int v = (e >= off) ? scan[e - off] : 0;
@@ -196,7 +205,12 @@ __global__ __launch_bounds__(1024) void sort_scan_kernel(int32_t* __restrict__ c
   if (e < E) {
     starts[e] = start;
     if (e == E - 1) starts[E] = scan[e];
-    for (int c = 0; c < nchunks; ++c) chunk_hist[(int64_t)c * E + e] += start;
+    int run = start;
+    for (int c = 0; c < nchunks; ++c) {
+      const int v = chunk_hist[(int64_t)c * E + e];
+      chunk_hist[(int64_t)c * E + e] = run;
+      run += v;
+    }
   }
 }
 
@@ -449,8 +463,8 @@ int64_t pk_sort_workspace_bytes(int64_t A, int64_t E) {
 }
 
 int pk_sort_by_expert(const int32_t* top_idx, int64_t A, int64_t E, int32_t* counts,
-                      int32_t* starts, int32_t* perm, int32_t* inv_perm, void* workspace,
-                      int64_t workspace_bytes, pk_stream_t stream) {
+                      int32_t* starts, int32_t* perm, int32_t* inv_perm, int32_t* order,
+                      void* workspace, int64_t workspace_bytes, pk_stream_t stream) {
   if (A < 0 || E <= 0) return PK_ERR_ARG;
   if (E > PK_MAX_EXPERTS || A > 0x7fffffffll) return PK_ERR_SHAPE;
   if (!starts || !workspace || (A > 0 && (!top_idx || !perm))) return PK_ERR_ARG;
@@ -463,7 +477,7 @@ int pk_sort_by_expert(const int32_t* top_idx, int64_t A, int64_t E, int32_t* cou
                      chunk_hist);
   PK_RETURN_IF_LAUNCH_FAILED();
   PK_LAUNCH_NOCHECK(pk_timing::K_SORT_SCAN, s, sort_scan_kernel, dim3(1), dim3(1024), 0, s, chunk_hist, nchunks, (int)E,
-                     counts, starts);
+                     counts, starts, order);
   PK_RETURN_IF_LAUNCH_FAILED();
   if (A > 0) {
     PK_LAUNCH_NOCHECK(pk_timing::K_SORT_SCATTER, s, sort_scatter_kernel, dim3(nchunks), dim3(64), lds, s, top_idx, (int)A,

@@ -200,16 +200,16 @@ class _ExpertRegionFn(torch.autograd.Function):
         E = w1.shape[0]
         logits = ops.gate_logits(x, w_gate, gate_bias)
         top_scores, top_idx = ops.route_topk(logits, top_k, route_norm, route_scale)
-        _counts, starts, perm, inv_perm = ops.sort_by_expert(top_idx, E)
+        _counts, starts, perm, inv_perm, order = ops.sort_by_expert(top_idx, E, with_order=True)
         y, g, u, h = ops.grouped_swiglu_fwd(x, w1, w2, w3, starts, row_map=perm, row_map_div=top_k)
         out = ops.combine_fwd(y, inv_perm, top_scores)
-        ctx.save_for_backward(x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, h, y)
+        ctx.save_for_backward(x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, h, y, order)
         ctx.cfg = (top_k, route_norm, route_scale, gate_bias is not None)
         return out
 
     @staticmethod
     def backward(ctx, d_out):
-        (x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, h, y) = ctx.saved_tensors
+        (x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, h, y, order) = ctx.saved_tensors
         top_k, route_norm, route_scale, has_bias = ctx.cfg
         E = w1.shape[0]
         need = ctx.needs_input_grad
@@ -224,9 +224,9 @@ class _ExpertRegionFn(torch.autograd.Function):
             if side is not None:
                 side.wait_stream(cur)
                 with torch.cuda.stream(side):
-                    d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k)
+                    d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k, expert_order=order)
             else:
-                d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k)
+                d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k, expert_order=order)
         d_xs = ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
         d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
         d_wg = torch.empty_like(w_gate) if need[1] else None

@@ -81,9 +81,10 @@ def route_topk_bwd(logits, top_idx, d_top_scores, route_norm: bool, route_scale:
     return d_logits
 
 
-def sort_by_expert(top_idx: torch.Tensor, num_experts: int):
+def sort_by_expert(top_idx: torch.Tensor, num_experts: int, with_order: bool = False):
     """Stable counting sort of the flat (token, k) slots by expert id.
-    Returns (counts [E], starts [E+1], perm [A], inv_perm [A]), all int32."""
+    Returns (counts [E], starts [E+1], perm [A], inv_perm [A]), all int32; with_order appends
+    order [E], the experts by descending row count (a scheduling hint for the weight gradient)."""
     require_gpu(top_idx)
     _check(top_idx.dtype == torch.int32, "sort_by_expert: top_idx must be int32")
     flat = top_idx.contiguous().view(-1)
@@ -97,8 +98,11 @@ def sort_by_expert(top_idx: torch.Tensor, num_experts: int):
     if ws_bytes < 0:
         raise RuntimeError(f"pk_sort_workspace_bytes failed: {_lib.status_string(ws_bytes)}")
     ws = torch.empty(max(int(ws_bytes), 4), dtype=torch.uint8, device=dev)
+    order = torch.empty(num_experts, dtype=torch.int32, device=dev) if with_order else None
     call("pk_sort_by_expert", ptr(flat), A, num_experts, ptr(counts), ptr(starts), ptr(perm), ptr(inv_perm),
-         ptr(ws), ws.numel(), current_stream(dev))
+         ptr(order), ptr(ws), ws.numel(), current_stream(dev))
+    if with_order:
+        return counts, starts, perm, inv_perm, order
     return counts, starts, perm, inv_perm
 
 
@@ -223,7 +227,7 @@ def grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts):
 
 
 def grouped_swiglu_wgrad(d_y, h, d_g, d_u, x_rows, starts, E, *, row_map=None, row_map_div=1,
-                         d_w1=None, d_w2=None, d_w3=None, accumulate=False):
+                         d_w1=None, d_w2=None, d_w3=None, accumulate=False, expert_order=None):
     """Weight gradients.  Without d_w* buffers, fresh tensors are returned; with buffers and
     accumulate=True the kernel adds into them (gradient accumulation over microbatches)."""
     require_gpu(d_y)
@@ -236,7 +240,7 @@ def grouped_swiglu_wgrad(d_y, h, d_g, d_u, x_rows, starts, E, *, row_map=None, r
         d_w3 = torch.empty((E, I, H), dtype=dt, device=dev)
         accumulate = False
     call("pk_grouped_swiglu_wgrad", ptr(d_y.contiguous()), ptr(h), ptr(d_g), ptr(d_u), ptr(x_rows.contiguous()),
-         ptr(row_map), row_map_div, ptr(starts), ptr(d_w1), ptr(d_w2), ptr(d_w3), int(bool(accumulate)),
+         ptr(row_map), row_map_div, ptr(starts), ptr(expert_order), ptr(d_w1), ptr(d_w2), ptr(d_w3), int(bool(accumulate)),
          A, H, I, E, dtype_code(dt), current_stream(dev))
     return d_w1, d_w2, d_w3
 

@@ -164,3 +164,14 @@ def test_end_to_end_routing_from_activations(dev):
     for r in diff_rows.tolist():
         assert gaps[r].min().item() < 1e-4, f"row {r} differs without a near-tie"
     assert len(diff_rows) <= 8
+
+
+def test_sort_expert_order_hint(dev):
+    """order = experts by descending row count, ties to the lower index."""
+    g = torch.Generator().manual_seed(3)
+    idx = torch.randint(0, 24, (500, 2), generator=g).int()
+    idx[idx == 7] = 3          # expert 7 empty, expert 3 popular
+    counts, starts, perm, inv, order = ops.sort_by_expert(idx.to(dev), 24, with_order=True)
+    c = counts.cpu().tolist()
+    expect = sorted(range(24), key=lambda e: (-c[e], e))
+    assert order.cpu().tolist() == expect and c[7] == 0 and expect[0] == 3
