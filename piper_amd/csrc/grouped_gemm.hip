@@ -1,12 +1,17 @@
 // Grouped SwiGLU expert GEMMs (forward, input gradient, weight gradient).
-//   bf16: v_mfma_f32_32x32x16_bf16 tiles, 128x128x64 block tile, 4 waves (2x2), fused
-//         SwiGLU / SwiGLU-backward epilogues, permute fused into the A-operand loader,
-//         ragged row blocks located on the device from starts[] (no host sync, empty
-//         experts launch nothing).
+//   bf16: v_mfma_f32_32x32x16_bf16 tiles fed by a ring of direct-to-LDS loads.
+//         Forward and input gradient: persistent workgroups (one per CU) that take
+//         (expert, row tile, column tile) units from per-XCD counters, 256x256x32 block tiles
+//         with 8 waves, fused SwiGLU / SwiGLU-backward epilogues, permute fused into the
+//         A-operand loader; ragged row tiles are located on the device from starts[] (no host
+//         sync).  Weight gradient: one workgroup per (expert, output tile), 256x256x64 tiles.
 //   f32 : tiled FMA kernel (simt_gemm.h) + elementwise SwiGLU kernels; exact fp32 arithmetic.
 #include "pk_common.h"
 #include "simt_gemm.h"
+#include <atomic>
+#include <cstdlib>
 #include <initializer_list>
+#include <mutex>
 
 namespace {
 
@@ -14,6 +19,7 @@ namespace {
 namespace mf {
 
 constexpr int NXCD = 8;
+
 
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_SWIGLU_BWD = 2 };
 
@@ -238,17 +244,42 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Ragged-M tile lookup, done redundantly by every wave (no LDS, no barrier).
-// Expert e owns ceil(cnt_e/BM) * n_tiles units, laid out [n-tile][m-tile] so that neighbouring
-// units share the weight tile.  Returns false when `unit` is past the last real tile.
+// Wait until at most `t` (0..MAXT) whole tiles of L loads each are still in flight.
+template <int L, int MAXT>
+__device__ __forceinline__ void wait_tiles(int t) {
+  if (MAXT <= 0 || t <= 0) { wait_dma<0>(); return; }
+  if (t >= MAXT) { wait_dma<(MAXT > 0 ? MAXT : 0) * L>(); return; }
+  wait_tiles<L, (MAXT > 0 ? MAXT - 1 : 0)>(t);
+}
+
+// Wait until at most n (wave-uniform, rounded down to a multiple of 4, capped at 60) vector-memory
+// operations are outstanding.  Loads, stores and atomics retire from the counter in issue
+// order, so with n = a lower bound of the operations issued AFTER the ones of interest this
+// waits for those without waiting for the younger ones (for example an epilogue's stores).
+__device__ __forceinline__ void wait_vm_le(int n) {
+  switch ((n < 60 ? n : 60) >> 2) {
+    case 0: wait_dma<0>(); break;    case 1: wait_dma<4>(); break;    case 2: wait_dma<8>(); break;
+    case 3: wait_dma<12>(); break;   case 4: wait_dma<16>(); break;   case 5: wait_dma<20>(); break;
+    case 6: wait_dma<24>(); break;   case 7: wait_dma<28>(); break;   case 8: wait_dma<32>(); break;
+    case 9: wait_dma<36>(); break;   case 10: wait_dma<40>(); break;  case 11: wait_dma<44>(); break;
+    case 12: wait_dma<48>(); break;  case 13: wait_dma<52>(); break;  case 14: wait_dma<56>(); break;
+    default: wait_dma<60>(); break;
+  }
+}
+
+// Per-lane slice of the prefix sum of work units over experts: lane l covers experts
+// [l*epl, (l+1)*epl).  Built once per wave with ordinary loads; locating a unit afterwards
+// takes a ballot plus a short scalar walk, so it can run in the middle of the k-loop without
+// touching the vector-memory counter that tracks the LDS ring.
+struct UnitIndex {
+  int excl, incl, total, epl;
+};
 template <int BM>
-__device__ __forceinline__ bool locate_ragged_m(const int32_t* __restrict__ starts, int E,
-                                                int n_tiles, int unit, int& e_out, int& mt_out,
-                                                int& nt_out) {
+__device__ __forceinline__ UnitIndex build_unit_index(const int32_t* __restrict__ starts, int E, int n_tiles) {
   const int lane = threadIdx.x & 63;
-  const int epl = (E + 63) >> 6;
-  const int e_lo = lane * epl;
-  const int e_hi = min(E, e_lo + epl);
+  UnitIndex ui;
+  ui.epl = (E + 63) >> 6;
+  const int e_lo = lane * ui.epl, e_hi = min(E, e_lo + ui.epl);
   int mine = 0;
   for (int e = e_lo; e < e_hi; ++e) mine += ((starts[e + 1] - starts[e] + BM - 1) / BM) * n_tiles;
   int incl = mine;
@@ -257,25 +288,94 @@ __device__ __forceinline__ bool locate_ragged_m(const int32_t* __restrict__ star
     const int v = __shfl_up(incl, off, PK_WAVE);
     if (lane >= off) incl += v;
   }
-  const int excl = incl - mine;
-  const bool owner = unit >= excl && unit < incl;
-  const unsigned long long bal = __ballot(owner);
-  if (bal == 0ull) return false;
-  const int src = __ffsll((long long)bal) - 1;
-  int fe = 0, fmt = 0, fnt = 0;
-  if (owner) {
-    int u = unit - excl;
-    for (int e = e_lo; e < e_hi; ++e) {
-      const int tiles = (starts[e + 1] - starts[e] + BM - 1) / BM;
-      const int units = tiles * n_tiles;
-      if (u < units) { fe = e; fnt = u / tiles; fmt = u % tiles; break; }
-      u -= units;
-    }
+  ui.incl = incl;
+  ui.excl = incl - mine;
+  ui.total = __builtin_amdgcn_readlane(incl, 63);
+  return ui;
+}
+// unit < ui.total.  Units of expert e are laid out [n-tile][m-tile], so neighbouring units share
+// the weight tile.  Everything returned is wave-uniform.
+template <int BM>
+__device__ __forceinline__ void locate_unit(const UnitIndex& ui, const_i32_ptr starts, int E, int n_tiles,
+                                            int unit, int& e_out, int& mt_out, int& nt_out) {
+  const unsigned long long bal = __ballot(unit >= ui.excl && unit < ui.incl);
+  const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)bal) - 1);
+  int u = unit - __builtin_amdgcn_readlane(ui.excl, src);
+  int e = src * ui.epl;
+  const int e_hi = min(E, e + ui.epl);
+  int tiles = 1;
+  for (; e < e_hi; ++e) {
+    tiles = (starts[e + 1] - starts[e] + BM - 1) / BM;
+    const int units = tiles * n_tiles;
+    if (u < units) break;
+    u -= units;
   }
-  e_out = __shfl(fe, src, PK_WAVE);
-  mt_out = __shfl(fmt, src, PK_WAVE);
-  nt_out = __shfl(fnt, src, PK_WAVE);
-  return true;
+  tiles = tiles > 0 ? tiles : 1;
+  e_out = e;
+  nt_out = u / tiles;
+  mt_out = u - nt_out * tiles;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Work distribution of the persistent kernels.  Units are grouped in chunks of SCHED_CHUNK
+// consecutive units; chunk c belongs to XCD c % 8, whose workgroups take its units one at a
+// time from a counter, so the workgroups of an XCD always run neighbouring units (shared
+// operands stay in that XCD's L2) while uneven unit costs still balance.  A workgroup whose own
+// XCD has run dry takes units from the other XCDs' counters.  Every launch uses one slot of a
+// pool of counter sets; the last workgroup to finish zeroes the slot again, so no memset
+// precedes a launch and launches in flight on different streams do not share counters.
+constexpr int SCHED_CHUNK = 32;
+constexpr int SCHED_SLOTS = 1024;
+struct SchedSlot {
+  unsigned grabs[NXCD];
+  unsigned finished;
+  unsigned pad[7];
+};
+__device__ SchedSlot g_sched_pool[SCHED_SLOTS];
+
+__device__ __forceinline__ int sched_unit_of(unsigned j, int x) {
+  return (int)(((j / SCHED_CHUNK) * NXCD + x) * SCHED_CHUNK + j % SCHED_CHUNK);
+}
+// One lane: take the next grab index of XCD x.  The request and the wait for its answer are one
+// statement, so the compiler never sees a register whose value is still on its way; the wait
+// drains the whole vector-memory counter, so this goes where that counter is about to be
+// drained anyway (after the last store of an epilogue).
+__device__ __forceinline__ unsigned sched_grab(SchedSlot* slot, int x) {
+  unsigned ret;
+  const unsigned one = 1u;
+  asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)"
+               : "=&v"(ret) : "v"(&slot->grabs[x]), "v"(one) : "memory");
+  return ret;
+}
+// Publish a value in LDS for the other waves: the write must have landed before this wave
+// arrives at the next barrier, also on paths that issue no further LDS traffic.
+__device__ __forceinline__ void lds_publish(int* box, int v) {
+  *box = v;
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+}
+// One lane: the next unit for a workgroup of XCD `xcd` (own counter first, then the others), or
+// -1 when all units are taken.  `first` is an already fetched grab index of the own counter.
+__device__ __forceinline__ int sched_resolve(SchedSlot* slot, int xcd, unsigned first, int total) {
+  int unit = sched_unit_of(first, xcd);
+  if (unit < total) return unit;
+  for (int a = 1; a < NXCD; ++a) {
+    const int x = (xcd + a) % NXCD;
+    // skip counters that are visibly exhausted (plain read first keeps them from running away)
+    if (sched_unit_of(__atomic_load_n(&slot->grabs[x], __ATOMIC_RELAXED), x) >= total) continue;
+    unit = sched_unit_of(atomicAdd(&slot->grabs[x], 1u), x);
+    if (unit < total) return unit;
+  }
+  return -1;
+}
+// One lane, after the workgroup's last unit: the last workgroup of the grid resets the slot.
+__device__ __forceinline__ void sched_finish(SchedSlot* slot) {
+  __threadfence();
+  if (atomicAdd(&slot->finished, 1u) == gridDim.x - 1) {
+#pragma unroll
+    for (int i = 0; i < NXCD; ++i) slot->grabs[i] = 0u;
+    slot->finished = 0u;
+    __threadfence();
+  }
 }
 
 struct RaggedMParams {
@@ -299,198 +399,400 @@ struct RaggedMParams {
   bf16_t* O1;            //            SWIGLU: u;  SWIGLU_BWD: d_u
   bf16_t* O2;            //            SWIGLU: h
   int64_t ldc;
+  SchedSlot* sched;      // this launch's counters
 #ifdef PK_GEMM_DEBUG
   int32_t debug;         // 1: skip MFMAs, 2: skip loads, 4: skip stores
 #endif
 };
 
+// Wave-private staging of 32 rows x COLS bf16 of the output through LDS, so that global stores
+// are 16 bytes per lane and row-contiguous.  Rows are unpadded (COLS*2 bytes); the 16-byte
+// chunks of row r are XOR-swizzled with r so that a column of 8-byte deposits spreads over the banks.
+template <int COLS>
+struct Stage32 {
+  static constexpr int ROWB = COLS * 2, CH = ROWB / 16, BYTES = 32 * ROWB;
+  static_assert((CH & (CH - 1)) == 0 && CH >= 2, "power-of-two chunk count");
+  // a lane deposits 4 consecutive columns (col % 4 == 0) of one row
+  __device__ static __forceinline__ void put(char* buf, int row, int col, u32x2_t v) {
+    *reinterpret_cast<u32x2_t*>(buf + row * ROWB + ((((col >> 3) ^ row) & (CH - 1)) << 4) + (col & 7) * 2) = v;
+  }
+  // rows [0, nrows) go to dst[r * ldc + 0..COLS); returns the number of store instructions
+  // the wave issued (nrows is wave-uniform)
+  template <bool ACC>
+  __device__ static __forceinline__ int flush(const char* buf, bf16_t* dst, int64_t ldc, int nrows) {
+    constexpr int RPP = 64 / CH, NP = 32 / RPP;
+    const int lane = threadIdx.x & 63;
+    const int lr = lane / CH, lc = lane % CH;
+    u32x4_t v[NP];
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {     // all LDS reads first: one latency for the whole chunk
+      const int r = q * RPP + lr;
+      v[q] = *reinterpret_cast<const u32x4_t*>(buf + r * ROWB + (((lc ^ r) & (CH - 1)) << 4));
+    }
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      const int r = q * RPP + lr;
+      if (r < nrows) {
+        u32x4_t* g = reinterpret_cast<u32x4_t*>(dst + (int64_t)r * ldc + lc * 8);
+        if (ACC) {
+          const bf16x8_t a = __builtin_bit_cast(bf16x8_t, v[q]);
+          const bf16x8_t o = __builtin_bit_cast(bf16x8_t, *g);
+          bf16x8_t sum;
+#pragma unroll
+          for (int t = 0; t < 8; ++t) sum[t] = (bf16_t)((float)a[t] + (float)o[t]);
+          v[q] = __builtin_bit_cast(u32x4_t, sum);
+        }
+        *g = v[q];
+      }
+    }
+    return nrows >= 32 ? NP : nrows <= 0 ? 0 : (nrows + RPP - 1) / RPP;
+  }
+};
+
+// MFMAs of one BK-deep k-tile for a wave tile of TM x TN MFMA tiles, with the L direct-to-LDS
+// loads of a later tile spread evenly between them: a wave that issues its loads back to back
+// blocks on the memory pipeline for many hundred cycles with its MFMAs queued behind them.
+// Fragments are double buffered one 16-deep k-step ahead, and their LDS reads are spread between
+// the MFMAs as well, which keeps the LDS queue short while the ring is being written.  Operands are passed to the MFMA
+// swapped (B first) so that a lane's accumulator holds 4 CONSECUTIVE columns of ONE row:
+//   acc[i][j][v] = C[row = 32*i + lane%32][col = 32*j + 8*(v/4) + 4*(lane/32) + v%4]
+template <int BK, int TM, int TN, bool A_KC, bool B_KC, int ACOLS, int BCOLS, int L, typename F>
+__device__ __forceinline__ void mma_ktile(const char* At, const char* Bt, int wrow0, int wcol0,
+                                          floatx16_t (&acc)[TM][TN], bool do_issue, F&& issue_one) {
+  const int lane = threadIdx.x & 63;
+  constexpr int KS = BK / 16, NM = KS * TM * TN;
+  constexpr int EVERY = NM / L > 0 ? NM / L : 1;
+  static_assert(L <= NM, "more loads than MFMAs in a k-tile");
+  static_assert(TM + TN <= TM * TN, "one fragment read per MFMA slot");
+  Frags<TM, TN> f[2];
+  load_frags<BK, TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[0], At, Bt, wrow0, wcol0, 0, lane);
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[ks & 1].b[j], f[ks & 1].a[i], acc[i][j], 0, 0, 0);
+        // the sched barriers pin one fragment read of the next k-step (B first: the next
+        // k-step starts with row 0) and at most one load behind each MFMA
+        __builtin_amdgcn_sched_barrier(0);
+        const int m = i * TN + j;
+        if (ks + 1 < KS) {
+          if (m < TN)
+            f[(ks + 1) & 1].b[m] = B_KC ? frag_kc<BK>(Bt, wcol0 + 32 * m, ks + 1, lane) : frag_mn<BCOLS>(Bt, wcol0 + 32 * m, ks + 1, lane);
+          else if (m < TN + TM)
+            f[(ks + 1) & 1].a[m - TN] = A_KC ? frag_kc<BK>(At, wrow0 + 32 * (m - TN), ks + 1, lane)
+                                             : frag_mn<ACOLS>(At, wrow0 + 32 * (m - TN), ks + 1, lane);
+        }
+        const int idx = (ks * TM + i) * TN + j;
+        if (idx % EVERY == EVERY - 1 && idx / EVERY < L) {
+          if (do_issue) issue_one(idx / EVERY);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+  }
+}
+
 // C[rows_e, N] = A[rows_e, K] . op(B[e]) with B K-contiguous ([N,K]) or MN-contiguous ([K,N]).
-// Block tile BM x BN, WMW x WNW waves, NS-stage LDS ring filled by direct-to-LDS loads.
+// Persistent workgroups (one per CU): each walks a strided list of work units (expert, row tile,
+// column tile), all units of one XCD being neighbours so that they share operands in its L2.
+// Block tile BM x BN x BK, WMW x WNW waves, NS-stage LDS ring filled by direct-to-LDS loads;
+// the ring is separate from the output staging, so the first NS-1 k-tiles of the next unit are
+// requested before the epilogue of the current one, and the next unit's addresses (row map
+// lookups included) are resolved with scalar loads during the current k-loop.
 // EPI_SWIGLU: the BN tile rows are [32 gate | 32 up | 32 gate | 32 up ...] of BN/2 output
 // columns, so that a lane holds the gate and the up value of the same element.
-template <int BM, int BN, int BK, int WMW, int WNW, int NS, int OCC, bool B_KC, int EPI>
-__global__ __launch_bounds__(64 * WMW * WNW, OCC * WMW * WNW / 4) void ragged_m_kernel(const RaggedMParams p) {
-  constexpr int NTHREADS = 64 * WMW * WNW;
+template <int BM, int BN, int BK, int WMW, int WNW, int NS, bool B_KC, int EPI>
+__global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMParams p) {
+  constexpr int NW = WMW * WNW, NTHREADS = 64 * NW;
   constexpr int WTM = BM / WMW, WTN = BN / WNW;          // wave tile
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int A_BYTES = BM * BK * 2, STAGE = (BM + BN) * BK * 2;
-  constexpr int LA = A_BYTES / (NTHREADS * 16), LB = (STAGE - A_BYTES) / (NTHREADS * 16);   // dma16 per thread per tile
+  constexpr int LA = A_BYTES / (NTHREADS * 16), LB = (STAGE - A_BYTES) / (NTHREADS * 16), L = LA + LB;
   static_assert(LA >= 1 && LB >= 1 && TM >= 1 && TN >= 1, "tile too small for the wave grid");
   static_assert(EPI != EPI_SWIGLU || (WTN % 64 == 0), "gate/up pairs must stay inside a wave");
-  // output columns a wave writes per output tensor, and its staging buffer
-  constexpr int OUT_COLS = (EPI == EPI_SWIGLU) ? WTN / 2 : WTN;
-  using St = Stage<OUT_COLS>;
-  constexpr int STAGING = WTM * St::LD * (WMW * WNW);
-  constexpr int SMEM = STAGING > NS * STAGE ? STAGING : NS * STAGE;
-  __shared__ __attribute__((aligned(1024))) char smem[SMEM];
+  constexpr int OUT_COLS = (EPI == EPI_SWIGLU) ? WTN / 2 : WTN;   // columns a wave writes per output tensor
+  constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;       // output columns per tile
+  using St = Stage32<OUT_COLS>;
+  constexpr int RING = NS * STAGE;
+  static_assert(RING + NW * St::BYTES <= 160 * 1024, "LDS budget");
+  __shared__ __attribute__((aligned(1024))) char smem[RING + NW * St::BYTES];
+  constexpr int CPR = BK / 8, RPI = 64 / CPR;            // 16-byte chunks per A row, A rows per dma16
 
-  int e, mt, nt;
-  if (!locate_ragged_m<BM>(p.starts, p.E, p.n_tiles, logical_block(), e, mt, nt)) return;
-  const int row0 = p.starts[e] + mt * BM;
-  const int rows = min(BM, p.starts[e + 1] - row0);
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WNW, wn = wave % WNW;
-  const bool wave_has_rows = wm * WTM < rows;   // waves whose row slice is empty skip the math
+  char* const sbuf = smem + RING + wave * St::BYTES;
+  const const_i32_ptr starts = as_const(p.starts);
+  const const_i32_ptr row_map = as_const(p.row_map);
 
-  // ---- per-thread source pointers of the dma16 loads (k offset 0 of segment 0)
-  int64_t a_off[LA];
-#pragma unroll
-  for (int i = 0; i < LA; ++i) {
-    int r, kofs;
-    kc_slot<BK>(wave * LA + i, lane, r, kofs);
-    r = r < rows ? r : rows - 1;     // clamp: rows past the expert's range are never stored
-    int64_t src = row0 + r;
-    if (p.row_map) src = p.row_map[src] / p.map_div;
-    a_off[i] = src * p.lda + kofs;
+  // ---- first unit of this workgroup
+  // the next unit, written by one lane, double buffered; it lives in the first bytes of the
+  // staging area, which is idle between the first two barriers of a k-loop (nkt >= 2)
+  int* const sched_box = reinterpret_cast<int*>(smem + RING);
+  const UnitIndex ui = build_unit_index<BM>(p.starts, p.E, p.n_tiles);
+  const int xcd = blockIdx.x % NXCD;
+  unsigned grab = 0;                  // lane 0 of wave 0: grab index taken one unit ahead
+  if (tid == 0) {
+    const int first = sched_resolve(p.sched, xcd, sched_grab(p.sched, xcd), ui.total);
+    sched_box[0] = first;
+    if (first >= 0) grab = sched_grab(p.sched, xcd);
   }
-  int64_t b_off[LB];
+  __syncthreads();
+  int unit = __builtin_amdgcn_readfirstlane(sched_box[0]);
+  if (unit < 0) {
+    if (tid == 0) sched_finish(p.sched);
+    return;
+  }
+  int par = 0;
+
+  // ---- lane constants of the loaders
+  int a_kofs[LA];
+#pragma unroll
+  for (int i = 0; i < LA; ++i) { int r; kc_slot<BK>(wave * LA + i, lane, r, a_kofs[i]); }
+  int32_t b_loff[LB];     // element offset inside the expert's weight tile
   int b_mat[LB];
-  const int64_t b_base = (int64_t)e * p.strideB;
 #pragma unroll
   for (int i = 0; i < LB; ++i) {
     b_mat[i] = 0;
     if (B_KC) {
       int r, kofs;
       kc_slot<BK>(wave * LB + i, lane, r, kofs);
-      int n;
-      if (EPI == EPI_SWIGLU) {
-        b_mat[i] = (r >> 5) & 1;
-        n = nt * (BN / 2) + (r >> 6) * 32 + (r & 31);
-      } else {
-        n = nt * BN + r;
-      }
-      b_off[i] = b_base + (int64_t)n * p.ldb + kofs;
+      int n = r;
+      if (EPI == EPI_SWIGLU) { b_mat[i] = (r >> 5) & 1; n = (r >> 6) * 32 + (r & 31); }
+      b_loff[i] = (int32_t)(n * p.ldb + kofs);
     } else {
       int krow, cofs;
       mn_slot<BN>(wave * LB + i, lane, krow, cofs);
-      b_off[i] = b_base + (int64_t)krow * p.ldb + (int64_t)nt * BN + cofs;
+      b_loff[i] = (int32_t)(krow * p.ldb + cofs);
     }
   }
-
   const int kt_per_seg = p.Kseg / BK;
   const int nkt = kt_per_seg * p.nseg;
 
-  auto issue = [&](int kt, int stage) {
-    char* st = smem + stage * STAGE;
-    const int seg = kt >= kt_per_seg ? 1 : 0;
-    const int k0 = (kt - seg * kt_per_seg) * BK;
-    const bf16_t* A = seg ? p.A1 : p.A0;
-    const uint32_t a_lds = lds_addr(st) + (wave * LA) * 1024;
-    const uint32_t b_lds = lds_addr(st + A_BYTES) + (wave * LB) * 1024;
+  struct Unit {
+    int row0, rows, nt;
+    int64_t b_base;
+    int64_t a_off[LA];
+  };
+  auto setup = [&](Unit& t, int un) {
+    int e, mt, nt;
+    locate_unit<BM>(ui, starts, p.E, p.n_tiles, un, e, mt, nt);
+    const int s0 = starts[e], s1 = starts[e + 1];
+    t.row0 = s0 + mt * BM;
+    t.rows = min(BM, s1 - t.row0);
+    t.nt = nt;
+    t.b_base = (int64_t)e * p.strideB + (B_KC ? (int64_t)nt * BN_OUT * p.ldb : (int64_t)nt * BN);
 #pragma unroll
-    for (int i = 0; i < LA; ++i) dma16(A + a_off[i] + k0, a_lds + i * 1024);
+    for (int i = 0; i < LA; ++i) {
+      const int rbase = (wave * LA + i) * RPI;     // first tile row of this dma16 (wave-uniform)
+      int64_t src;
+      if (p.row_map) {
+        int sel = 0;
 #pragma unroll
-    for (int i = 0; i < LB; ++i) {
-      const bf16_t* B = (EPI == EPI_SWIGLU) ? (b_mat[i] ? p.B1 : p.B0) : (seg ? p.B1 : p.B0);
-      dma16(B + b_off[i] + (B_KC ? (int64_t)k0 : (int64_t)k0 * p.ldb), b_lds + i * 1024);
+        for (int r = 0; r < RPI; ++r) {
+          const int rr = min(rbase + r, t.rows - 1);   // rows past the range are never stored
+          const int m = row_map[t.row0 + rr];
+          if (lane / CPR == r) sel = m;
+        }
+        src = sel / p.map_div;
+      } else {
+        src = t.row0 + min(rbase + lane / CPR, t.rows - 1);
+      }
+      t.a_off[i] = src * p.lda + a_kofs[i];
     }
   };
 
-  floatx16_t acc[TM][TN];
+  // DMA of k-tile `kt` of unit `t` into ring stage `stage`: piece 0..LA-1 = A, LA..L-1 = B
+  int is_k0 = 0, is_seg = 0;
+  uint32_t is_a = 0, is_b = 0;
+  auto issue_setup = [&](int kt, int stage) {
+    is_seg = kt >= kt_per_seg ? 1 : 0;
+    is_k0 = (kt - is_seg * kt_per_seg) * BK;
+    is_a = lds_addr(smem + stage * STAGE) + (wave * LA) * 1024;
+    is_b = lds_addr(smem + stage * STAGE + A_BYTES) + (wave * LB) * 1024;
+  };
+  auto issue_piece = [&](const Unit& t, int piece) {
+    if (piece < LA) {
+      const bf16_t* A = is_seg ? p.A1 : p.A0;
+      dma16(A + t.a_off[piece] + is_k0, is_a + piece * 1024);
+    } else {
+      const int i = piece - LA;
+      const bf16_t* B = (EPI == EPI_SWIGLU) ? (b_mat[i] ? p.B1 : p.B0) : (is_seg ? p.B1 : p.B0);
+      dma16(B + t.b_base + b_loff[i] + (B_KC ? (int64_t)is_k0 : (int64_t)is_k0 * p.ldb), is_b + i * 1024);
+    }
+  };
+  auto issue_tile = [&](const Unit& t, int kt, int stage) {
+    issue_setup(kt, stage);
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    for (int i = 0; i < L; ++i) issue_piece(t, i);
+  };
+#ifdef PK_GEMM_DEBUG
+  const bool dbg_loads = !(p.debug & 2), dbg_mma = !(p.debug & 1);
+#else
+  constexpr bool dbg_loads = true, dbg_mma = true;
+#endif
 
+  int st_after = 0;     // stores this wave issued after its latest prefetch
+  Unit cur_u, nxt_u;
+  setup(cur_u, unit);
+  nxt_u = cur_u;
+  int cur = 0;          // ring stage of k-tile 0 of the current unit
 #pragma unroll
   for (int s = 0; s < NS - 1; ++s)
-    if (s < nkt) issue(s, s);
-  int cur = 0;            // stage of tile kt
-  int nxt = NS - 1;       // stage of tile kt + NS - 1
-  for (int kt = 0; kt < nkt; ++kt) {
-    // tile kt has landed once at most the NS-2 younger tiles are still in flight
-    if (kt + NS - 2 < nkt) wait_dma<(NS - 2) * (LA + LB)>(); else wait_dma<0>();
-    block_barrier();   // everyone's part of tile kt is in LDS; everyone is done reading tile kt-1
-#ifdef PK_GEMM_DEBUG
-    if (!(p.debug & 2))
-#endif
-    if (kt + NS - 1 < nkt) issue(kt + NS - 1, nxt);
-    const char* st = smem + cur * STAGE;
-#ifdef PK_GEMM_DEBUG
-    if (!(p.debug & 1))
-#endif
-    if (wave_has_rows)
-      mma_tile<BK, TM, TN, true, B_KC, BM, BN, false>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
-    cur = cur + 1 == NS ? 0 : cur + 1;
-    nxt = nxt + 1 == NS ? 0 : nxt + 1;
-  }
-#ifdef PK_GEMM_DEBUG
-  if (p.debug & 4) { if (acc[0][0][0] != 12345.678f) return; }
-#endif
+    if (s < nkt && dbg_loads) issue_tile(cur_u, s, s);
 
-  // ---- epilogue: stage each wave's tile through LDS, then 16-byte row-contiguous stores
-  block_barrier();   // the ring is free: every wave has finished its last fragment reads
-  if (!wave_has_rows) return;
-  char* sbuf = smem + wave * (WTM * St::LD);
-  const int lrow = lane & 31, lq = 4 * (lane >> 5);
-  const int wrows = min(WTM, rows - wm * WTM);          // valid rows of this wave's slice
-  const int64_t grow0 = (int64_t)(row0 + wm * WTM) * p.ldc;
-  if (EPI == EPI_SWIGLU) {
-    const int64_t gcol0 = (int64_t)nt * (BN / 2) + wn * OUT_COLS;
+  for (;;) {
+    int unit_next = -1;
+    const bool wave_has_rows = wm * WTM < cur_u.rows;   // waves whose row slice is empty skip the math
+
+    floatx16_t acc[TM][TN];
 #pragma unroll
-    for (int which = 0; which < 3; ++which) {
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int j = 0; j < TN; j += 2)
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    for (int kt = 0; kt < nkt; ++kt) {
+      // k-tile kt has landed once only younger operations are in flight: the younger k-tiles
+      // and, before k-tile 0, the stores that the previous epilogue issued after its prefetch
+      if (kt == 0) wait_vm_le(min(NS - 2, nkt - 1) * L + st_after);
+      else wait_tiles<L, NS - 2>(min(NS - 2, nkt - 1 - kt));
+      block_barrier();   // everyone's part of tile kt is in LDS; everyone is done reading tile kt-1
+      if (kt == 0 && tid == 0)         // publish the unit after this one
+        lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, ui.total));
+      if (kt == 1) {                    // the box was written before this k-tile's barrier
+        unit_next = __builtin_amdgcn_readfirstlane(sched_box[par ^ 1]);
+        if (unit_next >= 0) setup(nxt_u, unit_next);
+      }
+      const int tgt = cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1;   // stage of k-tile kt-1 = kt+NS-1
+      issue_setup(kt + NS - 1, tgt);
+      const bool do_issue = dbg_loads && kt + NS - 1 < nkt;
+      const char* st = smem + cur * STAGE;
+      if (wave_has_rows && dbg_mma) {
+        mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, wm * WTM, wn * WTN, acc, do_issue,
+                                                     [&](int piece) { issue_piece(cur_u, piece); });
+      } else if (do_issue) {
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const u32x2_t gp = pack4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-            const u32x2_t up = pack4(acc[i][j + 1][4 * q], acc[i][j + 1][4 * q + 1], acc[i][j + 1][4 * q + 2], acc[i][j + 1][4 * q + 3]);
-            u32x2_t v = which == 0 ? gp : up;
-            if (which == 2) {
-              float g[4], u[4];
-              unpack4(gp, g);
-              unpack4(up, u);
-              v = pack4((g[0] / (1.f + __expf(-g[0]))) * u[0], (g[1] / (1.f + __expf(-g[1]))) * u[1],
-                        (g[2] / (1.f + __expf(-g[2]))) * u[2], (g[3] / (1.f + __expf(-g[3]))) * u[3]);
-            }
-            St::put(sbuf, 32 * i + lrow, 16 * j + 8 * q + lq, v);
-          }
-      wave_lds_fence();
-      bf16_t* dst = (which == 0 ? p.O0 : which == 1 ? p.O1 : p.O2) + grow0 + gcol0;
-      St::template flush<WTM>(sbuf, dst, p.ldc, wrows);
-      wave_lds_fence();
+        for (int i = 0; i < L; ++i) issue_piece(cur_u, i);
+      }
+      cur = cur + 1 == NS ? 0 : cur + 1;
     }
-  } else {
-    const int64_t gcol0 = (int64_t)nt * BN + wn * WTN;
+    block_barrier();   // every wave has finished its fragment reads: the whole ring is free
+    const bool has_next = unit_next >= 0;
+    // nothing is in flight here, so taking the ticket of the unit after the next one costs
+    // one round trip on one wave, not a drain of stores
+    if (has_next && tid == 0) grab = sched_grab(p.sched, xcd);
+
+    auto prefetch_next = [&]() {
+      st_after = 0;
+      if (has_next) {
 #pragma unroll
-    for (int which = 0; which < (EPI == EPI_PLAIN ? 1 : 2); ++which) {
+        for (int s = 0; s < NS - 1; ++s)
+          if (s < nkt && dbg_loads) issue_tile(nxt_u, s, cur + s >= NS ? cur + s - NS : cur + s);
+      }
+    };
+    if (EPI != EPI_SWIGLU_BWD) prefetch_next();
+
+    // ---- epilogue, 32 rows of the wave tile at a time through the wave's staging buffer
+    const int lrow = lane & 31, lq = 4 * (lane >> 5);
+    const int64_t grow0 = (int64_t)(cur_u.row0 + wm * WTM) * p.ldc;
+    const int64_t gcol0 = (int64_t)cur_u.nt * BN_OUT + wn * OUT_COLS;
+#ifdef PK_GEMM_DEBUG
+    const bool do_store = !(p.debug & 4);
+#else
+    constexpr bool do_store = true;
+#endif
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int r = 32 * i + lrow;
+    for (int i = 0; i < TM; ++i) {
+      const int crows = min(32, cur_u.rows - wm * WTM - 32 * i);   // valid rows of this chunk
+      const int64_t goff = grow0 + (int64_t)(32 * i) * p.ldc + gcol0;
+      if (EPI == EPI_SWIGLU) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int which = 0; which < 3; ++which) {
+          if (crows > 0 && do_store) {
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int c = 32 * j + 8 * q + lq;
-            u32x2_t v = pack4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-            if (EPI == EPI_SWIGLU_BWD) {   // acc = d_h (rounded to bf16 like the reference's bmm output)
-              float dh[4], g[4], u[4], o[4];
-              unpack4(v, dh);
-              const int rr = r < wrows ? r : wrows - 1;
-              const int64_t off = grow0 + (int64_t)rr * p.ldc + gcol0 + c;
+            for (int j = 0; j < TN; j += 2)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                const u32x2_t gp = pack4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+                const u32x2_t up = pack4(acc[i][j + 1][4 * q], acc[i][j + 1][4 * q + 1], acc[i][j + 1][4 * q + 2], acc[i][j + 1][4 * q + 3]);
+                u32x2_t v = which == 0 ? gp : up;
+                if (which == 2) {
+                  float g[4], u[4];
+                  unpack4(gp, g);
+                  unpack4(up, u);
+                  v = pack4((g[0] / (1.f + __expf(-g[0]))) * u[0], (g[1] / (1.f + __expf(-g[1]))) * u[1],
+                            (g[2] / (1.f + __expf(-g[2]))) * u[2], (g[3] / (1.f + __expf(-g[3]))) * u[3]);
+                }
+                St::put(sbuf, lrow, 16 * j + 8 * q + lq, v);
+              }
+            wave_lds_fence();
+            st_after += St::template flush<false>(sbuf, (which == 0 ? p.O0 : which == 1 ? p.O1 : p.O2) + goff, p.ldc, crows);
+            wave_lds_fence();
+          }
+        }
+      } else if (EPI == EPI_PLAIN) {
+        if (crows > 0 && do_store) {
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              St::put(sbuf, lrow, 32 * j + 8 * q + lq,
+                      pack4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]));
+          wave_lds_fence();
+          st_after += St::template flush<false>(sbuf, p.O0 + goff, p.ldc, crows);
+          wave_lds_fence();
+        }
+      } else {   // EPI_SWIGLU_BWD: acc = d_h; d_g = d_h * u * silu'(g), d_u = d_h * silu(g)
+        u32x2_t dg[TN][4], du[TN][4];
+        if (crows > 0) {
+          const int rr = lrow < crows ? lrow : crows - 1;
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int64_t off = goff + (int64_t)rr * p.ldc + 32 * j + 8 * q + lq;
+              float dh[4], g[4], u[4], og[4], ou[4];
+              // d_h is rounded to bf16 first, like the output of the reference's batched matmul
+              unpack4(pack4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]), dh);
               unpack4(*reinterpret_cast<const u32x2_t*>(p.Gin + off), g);
               unpack4(*reinterpret_cast<const u32x2_t*>(p.Uin + off), u);
 #pragma unroll
               for (int t = 0; t < 4; ++t) {
                 const float sg = 1.f / (1.f + __expf(-g[t]));
-                o[t] = which == 0 ? dh[t] * u[t] * (sg * (1.f + g[t] * (1.f - sg))) : dh[t] * (g[t] * sg);
+                og[t] = dh[t] * u[t] * (sg * (1.f + g[t] * (1.f - sg)));
+                ou[t] = dh[t] * (g[t] * sg);
               }
-              v = pack4(o[0], o[1], o[2], o[3]);
+              dg[j][q] = pack4(og[0], og[1], og[2], og[3]);
+              du[j][q] = pack4(ou[0], ou[1], ou[2], ou[3]);
             }
-            St::put(sbuf, r, c, v);
+        }
+        // the loads above must have returned first: a load behind the prefetch waits for all of it
+        __builtin_amdgcn_sched_barrier(0);
+        if (i == TM - 1) prefetch_next();
+        if (crows > 0 && do_store) {
+#pragma unroll
+          for (int which = 0; which < 2; ++which) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) St::put(sbuf, lrow, 32 * j + 8 * q + lq, which == 0 ? dg[j][q] : du[j][q]);
+            wave_lds_fence();
+            st_after += St::template flush<false>(sbuf, (which == 0 ? p.O0 : p.O1) + goff, p.ldc, crows);
+            wave_lds_fence();
           }
+        }
       }
-      wave_lds_fence();
-      bf16_t* dst = (which == 0 ? p.O0 : p.O1) + grow0 + gcol0;
-      St::template flush<WTM>(sbuf, dst, p.ldc, wrows);
-      wave_lds_fence();
     }
+    if (!has_next) break;
+    cur_u = nxt_u;
+    unit = unit_next;
+    par ^= 1;
   }
+  if (tid == 0) sched_finish(p.sched);
 }
 
 // ---- weight gradient: C[e][M,N] (+)= A[rows_e, M]^T . B[rows_e, N], ragged reduction dim.
@@ -648,15 +950,53 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
 
 inline int round_up_xcd(int64_t n) { return (int)(pk_ceil_div(n, NXCD) * NXCD); }
 
-template <int BM, int BN, int BK, int WMW, int WNW, int NS, int OCC, bool B_KC, int EPI>
+// One workgroup per CU (the ring takes most of the LDS), a multiple of 8 so that every XCD
+// gets the same number of slots.
+inline int persistent_grid() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    cached = cus / NXCD * NXCD;
+    if (cached < NXCD) cached = NXCD;
+  }
+  return cached;
+}
+
+// Counter set for one launch on the current device (nullptr if the pool cannot be resolved).
+inline SchedSlot* sched_slot_for_launch() {
+  constexpr int MAX_DEV = 64;
+  static SchedSlot* base[MAX_DEV] = {};
+  static std::mutex mu;
+  static std::atomic<unsigned> seq{0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) return nullptr;
+  if (!base[dev]) {
+    std::lock_guard<std::mutex> lock(mu);
+    if (!base[dev]) {
+      void* ptr = nullptr;
+      if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_sched_pool)) != hipSuccess || !ptr) return nullptr;
+      base[dev] = (SchedSlot*)ptr;
+    }
+  }
+  return base[dev] + (seq.fetch_add(1) % SCHED_SLOTS);
+}
+
+template <int BM, int BN, int BK, int WMW, int WNW, int NS, bool B_KC, int EPI>
 int launch_ragged_m(RaggedMParams p, int64_t A_rows, int kernel_id, hipStream_t s) {
 #ifdef PK_GEMM_DEBUG
   { const char* d = getenv("PK_GEMM_DEBUG_MODE"); p.debug = d ? atoi(d) : 0; }
 #endif
   const int64_t max_units = (pk_ceil_div(A_rows, BM) + p.E) * p.n_tiles;
-  if (max_units > 0x7ffffff0ll) return PK_ERR_SHAPE;
-  PK_LAUNCH_NOCHECK(kernel_id, s, (ragged_m_kernel<BM, BN, BK, WMW, WNW, NS, OCC, B_KC, EPI>),
-                    dim3(round_up_xcd(max_units)), dim3(64 * WMW * WNW), 0, s, p);
+  if (max_units > 0x7ffffff0ll || p.ldb * (int64_t)(BN > BK ? BN : BK) > 0x7fffffffll) return PK_ERR_SHAPE;
+  if ((int64_t)p.Kseg * p.nseg < 2 * BK) return PK_ERR_SHAPE;   // the k-loop publishes the next unit in its second step
+  const int64_t grid = max_units < persistent_grid() ? round_up_xcd(max_units) : persistent_grid();
+  p.sched = sched_slot_for_launch();
+  if (!p.sched) return PK_ERR_UNSUPPORTED;
+  PK_LAUNCH_NOCHECK(kernel_id, s, (ragged_m_kernel<BM, BN, BK, WMW, WNW, NS, B_KC, EPI>),
+                    dim3((unsigned)grid), dim3(64 * WMW * WNW), 0, s, p);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
 }
@@ -723,8 +1063,11 @@ int simt_ragged_k(const void* A, int64_t lda, const int32_t* a_map, const void* 
 // for the ragged-M kernels, 256x256 with 8 waves (128x64 wave tiles) for the weight gradient.
 // (BM, BN, BK, waves M, waves N, stages, workgroups per CU)
 #ifndef PK_RM_CFG
-#define PK_RM_CFG 128, 256, 64, 2, 4, 3, 1
+#define PK_RM_CFG 256, 256, 32, 2, 4, 4
 #define PK_RM_BN 256
+/* same width, 128 rows: for launches with few 256-row units per workgroup */
+#define PK_RM_LOWM 128, 256, 32, 2, 4, 5
+#define PK_RM_LOWM_UNITS 3
 #endif
 #ifndef PK_WG_BIG
 #define PK_WG_BIG 256, 256, 64, 2, 4, 2     /* 8 waves, 128x64 wave tiles, 128 KB ring */
@@ -733,7 +1076,7 @@ int simt_ragged_k(const void* A, int64_t lda, const int32_t* a_map, const void* 
 #define PK_WG_SMALL 128, 128, 64, 2, 2, 3
 #define PK_WG_SMALL_THREADS 256
 
-#define PK_RM_ALT 128, 128, 64, 2, 2, 3, 1      /* output widths that are a multiple of 128 but not of 256 */
+#define PK_RM_ALT 128, 128, 64, 2, 2, 3      /* output widths that are a multiple of 128 but not of 256 */
 bool mfma_shape_ok(int64_t H, int64_t I) { return H % 128 == 0 && I % 128 == 0; }
 
 // Pick the tile width by the output width N of the GEMM (for the gate/up kernel a tile holds
@@ -743,6 +1086,11 @@ int launch_rm(mf::RaggedMParams& p, int64_t A, int64_t N, int kernel_id, hipStre
   const int64_t per_tile_big = (EPI == mf::EPI_SWIGLU) ? PK_RM_BN / 2 : PK_RM_BN;
   if (N % per_tile_big == 0) {
     p.n_tiles = (int32_t)(N / per_tile_big);
+    // 256-row tiles unless they would leave the persistent grid with only a few units per
+    // workgroup (then the last round of units runs on a half-empty chip)
+    const int64_t big_units = (A / 256 + p.E / 2) * p.n_tiles;
+    const bool lowm = big_units < (int64_t)PK_RM_LOWM_UNITS * mf::persistent_grid();
+    if (lowm) return mf::launch_ragged_m<PK_RM_LOWM, B_KC, EPI>(p, A, kernel_id, s);
     return mf::launch_ragged_m<PK_RM_CFG, B_KC, EPI>(p, A, kernel_id, s);
   }
   const int64_t per_tile_alt = (EPI == mf::EPI_SWIGLU) ? 64 : 128;
