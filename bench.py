@@ -51,6 +51,30 @@ def kernel_flops(cfg) -> dict:
     }
 
 
+def kernel_bytes(cfg) -> dict:
+    """Algorithmic HBM bytes of ONE launch of each GEMM kernel: every operand read once, every
+    result written once (bf16).  A = routed rows, T = tokens, E experts, H hidden, I intermediate."""
+    A, T, E, H, I = cfg.routed_rows, cfg.tokens, cfg.num_experts, cfg.hidden, cfg.inter
+    w = 2.0 * E * I * H          # one expert weight tensor
+    return {
+        "swiglu_gate_up": 2 * w + 2.0 * T * H + 3 * 2.0 * A * I,        # w1,w3 + x (each token once) -> g,u,h
+        "swiglu_down": w + 2.0 * A * I + 2.0 * A * H,                   # w2 + h -> y
+        "swiglu_dgrad_dh": w + 2.0 * A * H + 2 * 2.0 * A * I + 2 * 2.0 * A * I,   # w2 + d_y + g,u -> d_g,d_u
+        "swiglu_dgrad_dx": 2 * w + 2 * 2.0 * A * I + 2.0 * A * H,       # w1,w3 + d_g,d_u -> d_x rows
+        "swiglu_wgrad": 2.0 * A * H + 3 * 2.0 * A * I + 2.0 * T * H + 3 * w,      # d_y,h,d_g,d_u,x -> d_w1..3
+    }
+
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the cfg3 workload,
+# scaled by what the same counters read for a plain device copy of known size
+# (profiles/bench_cfg3_hbm_traffic.md).  None where no measurement is committed.
+MEASURED_TRAFFIC_BYTES = {
+    "cfg3-qwen3-30b-a3b": {
+        "swiglu_wgrad": (700 + 1196) * 1e6,
+    },
+}
+
+
 def bench_region(cfg, steps: int, warmup: int):
     import torch
 
@@ -223,7 +247,23 @@ def main():
     gemm_kernels = {k: v for k, v in kernels.items() if k in flops}
     dominant = max(gemm_kernels, key=lambda k: gemm_kernels[k]["ms_per_step"])
     dom = gemm_kernels[dominant]
-    achieved = flops[dominant] / (dom["avg_ms"] * 1e-3) / 1e12
+    nbytes = kernel_bytes(cfg)
+    # the roofline that bounds the kernel: below the ridge point (peak flops / peak bandwidth) of
+    # the published peaks, moving its algorithmic bytes takes longer than its algorithmic flops
+    intensity = flops[dominant] / nbytes[dominant]
+    ridge = MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+    traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name, {}).get(dominant)
+    if intensity < ridge:
+        achieved = nbytes[dominant] / (dom["avg_ms"] * 1e-3) / 1e9
+        roof = {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBS, "traffic": traffic}
+    else:
+        achieved = flops[dominant] / (dom["avg_ms"] * 1e-3) / 1e12
+        roof = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic}
+    roof.update({"flops_per_launch": flops[dominant], "bytes_per_launch": nbytes[dominant],
+                 "flops_per_byte": intensity, "avg_launch_ms": dom["avg_ms"],
+                 "tflops": flops[dominant] / (dom["avg_ms"] * 1e-3) / 1e12})
     result = {
         "metric": "expert-region fwd+bwd tokens/s",
         "value": tokens_per_s,
@@ -242,9 +282,7 @@ def main():
                    "tokens_per_step": cfg.tokens},
         "mfma_frac_of_peak_region": mfma_frac_region,
         "gemm_tflops_region": gemm_flops_step / (ms_per_step * 1e-3) / 1e12,
-        "roofline": {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
-                     "flops_per_launch": flops[dominant], "avg_launch_ms": dom["avg_ms"]},
+        "roofline": roof,
         "kernels_ms_per_step": {k: round(v["ms_per_step"], 4) for k, v in sorted(kernels.items(), key=lambda kv: -kv[1]["ms_per_step"])},
         "gemm_kernels_tflops": {k: round(flops[k] / (v["avg_ms"] * 1e-3) / 1e12, 1) for k, v in gemm_kernels.items()},
     }
