@@ -22,9 +22,26 @@ struct Params {
   int32_t accumulate;  // splits == 1: C += result
 };
 
+// Four consecutive elements of an operand as floats (16-byte / 8-byte load).
+template <typename T>
+__device__ __forceinline__ void load4(const T* p, float (&out)[4]);
+template <>
+__device__ __forceinline__ void load4<float>(const float* p, float (&out)[4]) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+}
+template <>
+__device__ __forceinline__ void load4<bf16_t>(const bf16_t* p, float (&out)[4]) {
+  const bf16x4_t v = *reinterpret_cast<const bf16x4_t*>(p);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) out[j] = (float)v[j];
+}
+
 // A_KC / B_KC: the operand's k index is the contiguous one in memory (coalesce along k),
-// otherwise coalesce along m / n.
-template <int WM, int WN, bool A_KC, bool B_KC, typename TA, typename TB>
+// otherwise coalesce along m / n.  VEC: every thread fetches 4 consecutive elements of the
+// contiguous index per load (the host checks extents, strides and alignment); without it
+// loads are scalar and any extent works.
+template <int WM, int WN, bool A_KC, bool B_KC, typename TA, typename TB, bool VEC>
 __global__ __launch_bounds__(64 * WM * WN) void kernel(const Params p) {
   constexpr int BM = 32 * WM, BN = 32 * WN, THREADS = 64 * WM * WN;
   __shared__ float As[BM * LDS_LD];
@@ -45,39 +62,56 @@ __global__ __launch_bounds__(64 * WM * WN) void kernel(const Params p) {
   for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 
   // register prefetch: the loads of tile k+1 are in flight while tile k is multiplied
-  constexpr int NA = BM * BK / THREADS, NB = BN * BK / THREADS;
-  float ra[NA], rb[NB];
+  constexpr int W = VEC ? 4 : 1;
+  constexpr int NA = BM * BK / (THREADS * W), NB = BN * BK / (THREADS * W);
+  static_assert(NA >= 1 && NB >= 1, "tile too small for the thread count");
+  float ra[NA][W], rb[NB][W];
+  // element (row = m or n index in the tile, k) of the idx-th load of a tile with R rows
+  auto slot = [](int idx, bool kc, int R, int& row, int& k) {
+    if (kc) { k = (idx % (BK / W)) * W; row = idx / (BK / W); }
+    else { row = (idx % (R / W)) * W; k = idx / (R / W); }
+  };
   auto load_tile = [&](int64_t k0) {
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-      const int idx = tid + i * THREADS;
-      const int k = A_KC ? idx % BK : idx / BM;
-      const int m = A_KC ? idx / BK : idx % BM;
-      float v = 0.f;
-      if (m0 + m < p.M && k0 + k < kend) v = pk_to_float<TA>(A[(m0 + m) * p.sam + (k0 + k) * p.sak]);
-      ra[i] = v;
+      int m, k;
+      slot(tid + i * THREADS, A_KC, BM, m, k);
+#pragma unroll
+      for (int j = 0; j < W; ++j) ra[i][j] = 0.f;
+      if (m0 + m < p.M && k0 + k < kend) {
+        const TA* src = A + (m0 + m) * p.sam + (k0 + k) * p.sak;
+        if (VEC) load4<TA>(src, reinterpret_cast<float(&)[4]>(ra[i]));
+        else ra[i][0] = pk_to_float<TA>(*src);
+      }
     }
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-      const int idx = tid + i * THREADS;
-      const int k = B_KC ? idx % BK : idx / BN;
-      const int n = B_KC ? idx / BK : idx % BN;
-      float v = 0.f;
-      if (n0 + n < p.N && k0 + k < kend) v = pk_to_float<TB>(B[(k0 + k) * p.sbk + (n0 + n) * p.sbn]);
-      rb[i] = v;
+      int n, k;
+      slot(tid + i * THREADS, B_KC, BN, n, k);
+#pragma unroll
+      for (int j = 0; j < W; ++j) rb[i][j] = 0.f;
+      if (n0 + n < p.N && k0 + k < kend) {
+        const TB* src = B + (k0 + k) * p.sbk + (n0 + n) * p.sbn;
+        if (VEC) load4<TB>(src, reinterpret_cast<float(&)[4]>(rb[i]));
+        else rb[i][0] = pk_to_float<TB>(*src);
+      }
     }
   };
   if (kbeg < kend) load_tile(kbeg);
   for (int64_t k0 = kbeg; k0 < kend; k0 += BK) {
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-      const int idx = tid + i * THREADS;
-      As[(A_KC ? idx / BK : idx % BM) * LDS_LD + (A_KC ? idx % BK : idx / BM)] = ra[i];
+      int m, k;
+      slot(tid + i * THREADS, A_KC, BM, m, k);
+#pragma unroll
+      for (int j = 0; j < W; ++j) As[(A_KC ? m : m + j) * LDS_LD + (A_KC ? k + j : k)] = ra[i][j];
     }
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-      const int idx = tid + i * THREADS;
-      Bs[(B_KC ? idx / BK : idx % BN) * LDS_LD + (B_KC ? idx % BK : idx / BN)] = rb[i];
+      int n, k;
+      slot(tid + i * THREADS, B_KC, BN, n, k);
+#pragma unroll
+      for (int j = 0; j < W; ++j) Bs[(B_KC ? n : n + j) * LDS_LD + (B_KC ? k + j : k)] = rb[i][j];
     }
     __syncthreads();
     if (k0 + BK < kend) load_tile(k0 + BK);
@@ -118,12 +152,24 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
   out[i] = s;
 }
 
+// Whether every 4-element group along the contiguous index of an operand can be fetched with one
+// aligned load: extent and the other stride multiples of 4, base aligned to 4 elements.
+template <typename T>
+inline bool vec4_ok(const void* base, int64_t contig_extent, int64_t other_stride) {
+  return contig_extent % 4 == 0 && other_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(base) % (4 * sizeof(T))) == 0;
+}
+
 template <int WM, int WN, bool A_KC, bool B_KC, typename TA, typename TB>
 inline int launch(const Params& p, int kernel_id, hipStream_t s) {
   if (p.M <= 0 || p.N <= 0) return PK_OK;
   dim3 grid((unsigned)pk_ceil_div(p.N, 32 * WN), (unsigned)pk_ceil_div(p.M, 32 * WM), (unsigned)p.splits);
   if (grid.y > 65535u || grid.z > 65535u) return PK_ERR_SHAPE;
-  PK_LAUNCH_NOCHECK(kernel_id, s, (kernel<WM, WN, A_KC, B_KC, TA, TB>), grid, dim3(64 * WM * WN), 0, s, p);
+  const bool vec = (A_KC ? (p.sak == 1 && vec4_ok<TA>(p.A, p.K, p.sam)) : (p.sam == 1 && vec4_ok<TA>(p.A, p.M, p.sak))) &&
+                   (B_KC ? (p.sbk == 1 && vec4_ok<TB>(p.B, p.K, p.sbn)) : (p.sbn == 1 && vec4_ok<TB>(p.B, p.N, p.sbk)));
+  if (vec)
+    PK_LAUNCH_NOCHECK(kernel_id, s, (kernel<WM, WN, A_KC, B_KC, TA, TB, true>), grid, dim3(64 * WM * WN), 0, s, p);
+  else
+    PK_LAUNCH_NOCHECK(kernel_id, s, (kernel<WM, WN, A_KC, B_KC, TA, TB, false>), grid, dim3(64 * WM * WN), 0, s, p);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
 }

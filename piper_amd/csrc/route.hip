@@ -306,8 +306,8 @@ const char* pk_status_string(int status) {
 }
 
 static int gate_fwd_splits(int64_t H) {
-  int64_t sp = H / 512;
-  return (int)(sp < 1 ? 1 : (sp > 4 ? 4 : sp));
+  int64_t sp = H / 256;
+  return (int)(sp < 1 ? 1 : (sp > 8 ? 8 : sp));
 }
 
 int64_t pk_gate_workspace_bytes(int64_t T, int64_t H, int64_t E) {
@@ -354,8 +354,8 @@ int pk_gate_logits(const void* x, int x_dtype, const float* w_gate, const float*
 }
 
 static int gate_bwd_splits(int64_t T) {
-  int64_t sp = T / 512;
-  return (int)(sp < 1 ? 1 : (sp > 8 ? 8 : sp));
+  int64_t sp = T / 256;
+  return (int)(sp < 1 ? 1 : (sp > 16 ? 16 : sp));
 }
 
 int64_t pk_gate_bwd_workspace_bytes(int64_t T, int64_t H, int64_t E) {
