@@ -15,7 +15,9 @@ from typing import Any, Sequence
 
 import torch
 
+from . import functional as F_
 from .bucket import ParamStorage, StageStore
+from .planner import plan_zero_lifetimes
 from .tasks import COMM_TASKS, TaskType
 
 
@@ -114,6 +116,7 @@ class StageExecutor:
     loss_fn: Any = None
     _fwd: dict = field(default_factory=dict)
     _inp_grads: dict = field(default_factory=dict)
+    _wgrad_queues: dict = field(default_factory=dict)
 
     def __post_init__(self):
         self.params = self.params or ParamStorage(self.stages)
@@ -127,6 +130,7 @@ class StageExecutor:
         ps = self.pack_stream or cs
         self._fwd.clear()
         self._inp_grads.clear()
+        self._wgrad_queues.clear()
         losses = []
         pack_events: dict = {}
         self.params.clear_param_grads()
@@ -134,8 +138,11 @@ class StageExecutor:
         if ps is not cs:
             cs.wait_stream(ps)
         ubids = list(self.stages.buckets.keys())
-        for task in tasks:
+        # which task gathers / frees a bucket's parameters and which one packs its gradients
+        lifetimes = plan_zero_lifetimes(tasks)
+        for ti, task in enumerate(tasks):
             tt = task.type
+            life = lifetimes.get(ti)
             if tt in COMM_TASKS or tt is TaskType.ORDER_DUMMY:
                 continue
             if tt is TaskType.FWD:
@@ -144,48 +151,77 @@ class StageExecutor:
                     inp = microbatches[task.mb]
                 else:
                     inp = self._fwd[(ubids[pos - 1], task.mb)]["detached_outs"]
-                if task.ubid in self.stages.param_sharded_ubids:
+                if task.ubid in self.stages.param_sharded_ubids and life.gather_params_before:
                     self.params.all_gather_full_params(task.ubid, cs)
                 self._fwd[(task.ubid, task.mb)] = self.compute.forward(task.ubid, inp, cs)
-            elif tt in (TaskType.BWD, TaskType.FWD_BWD):
+                if task.ubid in self.stages.param_sharded_ubids and life.free_params_after:
+                    self.params.free_full_params(task.ubid)
+            elif tt in (TaskType.BWD, TaskType.FWD_BWD, TaskType.BWD_I):
+                # BWD_I is the same walk with the weight gradients of the HIP operators queued
+                # instead of computed (src/executors.py:353-411); BWD_W runs the queue (:413-476)
+                split = tt is TaskType.BWD_I
                 pos = ubids.index(task.ubid)
                 rec = self._fwd.pop((task.ubid, task.mb))
-                if pos == len(ubids) - 1:
-                    with torch.cuda.stream(cs):
-                        out = rec["pre_detach_outs"][0]
-                        if self.loss_fn is not None:
-                            loss = self.loss_fn(out, None if targets is None else targets[task.mb])
-                        else:
-                            loss = out.float().sum()
-                    losses.append(loss.detach())
-                    self.compute.backward(task.ubid, task.mb, [loss], None, None, None,
-                                          rec["inp_with_grad"], rec["out_with_grad"], cs)
-                else:
-                    # the downstream bucket's input grads become the grads of this bucket's detached
-                    # outputs (src/executors.py:826-842)
-                    prev = self._inp_grads.pop((ubids[pos + 1], task.mb))
-                    for d, g in zip(rec["detached_outs"], prev):
-                        if isinstance(d, torch.Tensor) and d.requires_grad and g is not None:
-                            d.grad = g
-                    self.compute.backward(task.ubid, task.mb, rec["pre_detach_outs"], None, rec["pre_detach_outs"],
-                                          rec["detached_outs"], rec["inp_with_grad"], rec["out_with_grad"], cs)
+                if task.ubid in self.stages.param_sharded_ubids and life.gather_params_before:
+                    self.params.all_gather_full_params(task.ubid, cs)
+                ctx = F_.defer_weight_grads() if split else None
+                queue = ctx.__enter__() if split else None
+                try:
+                    if pos == len(ubids) - 1:
+                        with torch.cuda.stream(cs):
+                            out = rec["pre_detach_outs"][0]
+                            if self.loss_fn is not None:
+                                loss = self.loss_fn(out, None if targets is None else targets[task.mb])
+                            else:
+                                loss = out.float().sum()
+                        losses.append(loss.detach())
+                        self.compute.backward(task.ubid, task.mb, [loss], None, None, None,
+                                              rec["inp_with_grad"], rec["out_with_grad"], cs)
+                    else:
+                        # the downstream bucket's input grads become the grads of this bucket's detached
+                        # outputs (src/executors.py:826-842)
+                        prev = self._inp_grads.pop((ubids[pos + 1], task.mb))
+                        for d, g in zip(rec["detached_outs"], prev):
+                            if isinstance(d, torch.Tensor) and d.requires_grad and g is not None:
+                                d.grad = g
+                        self.compute.backward(task.ubid, task.mb, rec["pre_detach_outs"], None, rec["pre_detach_outs"],
+                                              rec["detached_outs"], rec["inp_with_grad"], rec["out_with_grad"], cs)
+                finally:
+                    if split:
+                        ctx.__exit__(None, None, None)
                 self._inp_grads[(task.ubid, task.mb)] = [
                     t.grad if (isinstance(t, torch.Tensor) and t.requires_grad) else None for t in rec["fwd_inputs"]]
-                # gradient pack on the second stream, ordered after this backward
-                if ps is not cs:
-                    evt = torch.cuda.Event()
-                    evt.record(cs)
-                    ps.wait_event(evt)
-                self.params.accumulate_zero_param_grads_to_flat(task.ubid, ps if ps is not cs else None)
-                if ps is not cs:
-                    done = torch.cuda.Event()
-                    done.record(ps)
-                    pack_events[task.ubid] = done
+                if split:
+                    self._wgrad_queues[(task.ubid, task.mb)] = queue
+                if life.reduce_grads_after:
+                    self._pack_after_backward(task.ubid, cs, ps, pack_events)
+                if task.ubid in self.stages.param_sharded_ubids and life.free_params_after:
+                    self.params.free_full_params(task.ubid)
+            elif tt is TaskType.BWD_W:
+                queue = self._wgrad_queues.pop((task.ubid, task.mb))
+                with torch.cuda.stream(cs):
+                    queue.run()
+                if life.reduce_grads_after:
+                    self._pack_after_backward(task.ubid, cs, ps, pack_events)
+                if task.ubid in self.stages.param_sharded_ubids and life.free_params_after:
+                    self.params.free_full_params(task.ubid)
             elif tt is TaskType.UPD:
                 self._update(cs, pack_events)
             else:
-                raise NotImplementedError(f"task {tt} is scheduled through the split-backward operators, not this loop")
+                raise NotImplementedError(f"task {tt} is not a per-device task of this executor")
         return {"losses": losses}
+
+    def _pack_after_backward(self, ubid, cs, ps, pack_events: dict) -> None:
+        """Gradient pack on the second stream, ordered after the backward that produced the grads."""
+        if ps is not cs:
+            evt = torch.cuda.Event()
+            evt.record(cs)
+            ps.wait_event(evt)
+        self.params.accumulate_zero_param_grads_to_flat(ubid, ps if ps is not cs else None)
+        if ps is not cs:
+            done = torch.cuda.Event()
+            done.record(ps)
+            pack_events[ubid] = done
 
     def _update(self, stream, pack_events: dict):
         """src/executors.py:1005-1034."""

@@ -89,6 +89,7 @@ class _BmmExpertsFn(torch.autograd.Function):
         starts = ops.counts_to_starts(num_tokens_per_expert)
         y, g, u, h = ops.grouped_swiglu_fwd(x, w1, w2, w3, starts)
         ctx.save_for_backward(w1, w2, w3, x, starts, g, u, h)
+        ctx.params = (w1, w2, w3)
         return y
 
     @staticmethod
@@ -96,9 +97,31 @@ class _BmmExpertsFn(torch.autograd.Function):
         w1, w2, w3, x, starts, g, u, h = ctx.saved_tensors
         d_x, d_g, d_u = ops.grouped_swiglu_dgrad(d_y, w1, w2, w3, g, u, starts)
         d_w1 = d_w2 = d_w3 = None
-        if any(ctx.needs_input_grad[:3]):
+        if all(ctx.needs_input_grad[:3]) and _can_defer(*ctx.params):
+            _queue_expert_wgrad(ctx.params, d_y, h, d_g, d_u, x, starts, None, 1, None)
+        elif any(ctx.needs_input_grad[:3]):
             d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, w1.shape[0])
         return d_w1, d_w2, d_w3, d_x, None
+
+
+def _queue_expert_wgrad(params, d_y, h, d_g, d_u, x, starts, perm, top_k, order) -> None:
+    p1, p2, p3 = params
+
+    def run():
+        bufs = [_grad_target(p) for p in (p1, p2, p3)]
+        if all(acc for _, acc in bufs):     # accumulate in the kernel's epilogue
+            ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, p1.shape[0], row_map=perm, row_map_div=top_k,
+                                     expert_order=order, d_w1=bufs[0][0], d_w2=bufs[1][0], d_w3=bufs[2][0], accumulate=True)
+            return
+        g1, g2, g3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, p1.shape[0], row_map=perm,
+                                              row_map_div=top_k, expert_order=order)
+        for p, g in ((p1, g1), (p2, g2), (p3, g3)):
+            if p.grad is None:
+                p.grad = g
+            else:
+                p.grad += g
+
+    _WGRAD_QUEUE.push(run)
 
 
 def _bmm_experts_autograd(w1, w2, w3, x, num_tokens_per_expert):
@@ -168,6 +191,56 @@ def combine(gathered_output, token_indices_experts_sorted, top_scores):
     return _CombineFn.apply(gathered_output, token_indices_experts_sorted, top_scores)
 
 
+# --------------------------------------------------------------------------- split backward
+class WeightGradQueue:
+    """Weight-gradient work postponed by a backward-input pass (Piper's BWD_I / BWD_W split,
+    src/executors.py:353-476).  ``run()`` launches the postponed kernels and accumulates their
+    results into ``param.grad`` as the reference's weight pass does (src/executors.py:333-343)."""
+
+    def __init__(self):
+        self._work = []
+
+    def push(self, fn) -> None:
+        self._work.append(fn)
+
+    def __len__(self) -> int:
+        return len(self._work)
+
+    def run(self) -> None:
+        work, self._work = self._work, []
+        for fn in work:
+            fn()
+
+
+_WGRAD_QUEUE: WeightGradQueue | None = None
+
+
+class defer_weight_grads:
+    """Context manager: backward passes run inside it compute input gradients only; the weight
+    gradients of leaf parameters are queued on the returned WeightGradQueue."""
+
+    def __enter__(self) -> WeightGradQueue:
+        global _WGRAD_QUEUE
+        self._prev = _WGRAD_QUEUE
+        _WGRAD_QUEUE = WeightGradQueue()
+        return _WGRAD_QUEUE
+
+    def __exit__(self, *exc) -> None:
+        global _WGRAD_QUEUE
+        _WGRAD_QUEUE = self._prev
+
+
+def _can_defer(*params) -> bool:
+    return _WGRAD_QUEUE is not None and all(p is None or (p.is_leaf and p.requires_grad) for p in params)
+
+
+def _grad_target(p):
+    """(buffer to accumulate into, accumulate flag) for a leaf parameter."""
+    if p.grad is None:
+        return None, False
+    return p.grad, True
+
+
 # --------------------------------------------------------------------------- fused region
 # Measured on MI355X: running the weight gradient next to the input gradient gains ~1.5 % (both
 # kernels are throughput-bound), so it is opt-in; per-kernel timings are only meaningful with it off.
@@ -205,6 +278,7 @@ class _ExpertRegionFn(torch.autograd.Function):
         out = ops.combine_fwd(y, inv_perm, top_scores)
         ctx.save_for_backward(x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, h, y, order)
         ctx.cfg = (top_k, route_norm, route_scale, gate_bias is not None)
+        ctx.params = (w_gate, gate_bias, w1, w2, w3)
         return out
 
     @staticmethod
@@ -219,6 +293,33 @@ class _ExpertRegionFn(torch.autograd.Function):
         # second stream next to the input gradient (BWD_I) so the two kernels fill each other's tails.
         d_w1 = d_w2 = d_w3 = None
         cur = torch.cuda.current_stream(x.device)
+        defer = all(need[3:6]) and need[1] and _can_defer(*ctx.params)
+        if defer:
+            # backward-input pass: the weight gradients of the experts and of the router gate are
+            # queued with the tensors they need and computed by the weight pass
+            p_gate, p_bias = ctx.params[0], ctx.params[1]
+            _queue_expert_wgrad(ctx.params[2:], d_y, h, d_g, d_u, x, starts, perm, top_k, order)
+            d_xs = ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
+            d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
+            d_x32 = ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=need[0], d_w_gate=None, d_gate_bias=None)
+            d_x = ops.permute_bwd(d_xs, inv_perm, top_k, addend_f32=d_x32) if need[0] else None
+
+            def run_router():
+                acc = p_gate.grad is not None
+                gw = p_gate.grad if acc else torch.empty_like(p_gate)
+                gb = None
+                if p_bias is not None:
+                    if p_bias.grad is not None:
+                        gb = p_bias.grad if acc else p_bias.grad.clone()
+                    else:
+                        gb = torch.zeros_like(p_bias, dtype=torch.float32) if acc else torch.empty_like(p_bias, dtype=torch.float32)
+                ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=False, d_w_gate=gw, d_gate_bias=gb, accumulate=acc)
+                p_gate.grad = gw
+                if p_bias is not None:
+                    p_bias.grad = gb
+
+            _WGRAD_QUEUE.push(run_router)
+            return d_x, None, None, None, None, None, None, None, None
         side = _side_stream(x.device) if (need[3] or need[4] or need[5]) and _OVERLAP_WGRAD else None
         if need[3] or need[4] or need[5]:
             if side is not None:

@@ -47,13 +47,8 @@ def _oracle_iteration(layers, xs, dtype):
     return params, losses
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("two_streams", [True, False])
-def test_two_bucket_1f1b_iteration(dev, dtype, two_streams):
-    print(f"[case] executor {dtype} two_streams={two_streams}", flush=True)
-    layers, xs = _init(0, dtype)
-    ref_params, ref_losses = _oracle_iteration(layers, xs, dtype)
-
+def _make_executor(layers, xs, dev, dtype, two_streams):
+    """Two MoE layers as two compute buckets (+ fp32 gate buckets when the experts are bf16)."""
     store = StageStore()
     for ubid, l in enumerate(layers):
         b = BucketState()
@@ -90,11 +85,7 @@ def test_two_bucket_1f1b_iteration(dev, dtype, two_streams):
         store.zero_managed_ubids.add(name)
 
     compute_ubids = [0, 1]
-    tasks = one_f_one_b(MB, compute_ubids)
-    # gate buckets have no forward of their own: pack them right after their stage's backward
-    sched = []
-    for t in tasks:
-        sched.append(t)
+    # gate buckets have no forward of their own: they are packed right after their stage's backward
     ex = StageExecutor(store, compute_stream=torch.cuda.Stream() if two_streams else None,
                        pack_stream=torch.cuda.Stream() if two_streams else None)
     # the executor walks store.buckets in order for FWD chaining: restrict chaining to compute buckets
@@ -118,6 +109,18 @@ def test_two_bucket_1f1b_iteration(dev, dtype, two_streams):
             orig_acc(f"gate{ubid}", stream)
     ex.params.accumulate_zero_param_grads_to_flat = acc
 
+    return store, ex, mbs, compute_ubids
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("two_streams", [True, False])
+def test_two_bucket_1f1b_iteration(dev, dtype, two_streams):
+    print(f"[case] executor {dtype} two_streams={two_streams}", flush=True)
+    layers, xs = _init(0, dtype)
+    ref_params, ref_losses = _oracle_iteration(layers, xs, dtype)
+
+    store, ex, mbs, compute_ubids = _make_executor(layers, xs, dev, dtype, two_streams)
+    tasks = one_f_one_b(MB, compute_ubids)
     out = ex.run(tasks, mbs)
     torch.cuda.synchronize()
     tol = F32_TOL if dtype == torch.float32 else BF16_TOL
@@ -157,3 +160,59 @@ def test_comm_tasks_are_noops_and_unknown_bucket_raises(dev):
     assert out["losses"] == []
     with pytest.raises(KeyError):
         store.bucket("missing")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_split_backward_tasks_match_whole_backward(dev, dtype):
+    """BWD_I + BWD_W (src/executors.py:353-476) in a zero-bubble-like order give the same gradient
+    buckets and the same update as whole BWD tasks: the weight pass runs the same kernels later."""
+    print(f"[case] split backward {dtype}", flush=True)
+    layers, xs = _init(1, dtype)
+    results = []
+    for split in (False, True):
+        store, ex, mbs, ubids = _make_executor(layers, xs, dev, dtype, False)
+        tasks = []
+        for mb in range(MB):
+            tasks += [Task(TaskType.FWD, u, mb) for u in ubids]
+            if split:   # all input gradients first, then the weight gradients (any order is allowed)
+                tasks += [Task(TaskType.BWD_I, u, mb) for u in reversed(ubids)]
+                tasks += [Task(TaskType.BWD_W, u, mb) for u in ubids]
+            else:
+                tasks += [Task(TaskType.BWD, u, mb) for u in reversed(ubids)]
+        tasks.append(Task(TaskType.UPD))
+        out = ex.run(tasks, mbs)
+        torch.cuda.synchronize()
+        results.append((out["losses"], {u: (store.buckets[u].flat_grads.clone(), store.buckets[u].flat_params.clone())
+                                        for u in store.buckets}))
+    (l0, b0), (l1, b1) = results
+    for a, b in zip(l0, l1):
+        assert torch.equal(a, b)
+    for u in b0:
+        assert torch.equal(b0[u][0], b1[u][0]), f"gradient bucket {u}"
+        assert torch.equal(b0[u][1], b1[u][1]), f"parameter bucket {u}"
+
+
+def test_weight_grad_queue_accumulates_into_existing_grads(dev):
+    """Without packing in between, the weight pass adds to .grad like the reference's weight pass."""
+    layers, xs = _init(2, torch.float32)
+    l = layers[0]
+    ps = {k: torch.nn.Parameter(l[k].to(dev)) for k in NAMES}
+    x = xs[0].to(dev)
+
+    def run(deferred):
+        for p in ps.values():
+            p.grad = None
+        for _ in range(2):
+            out = F_.expert_region(x, ps["w_gate"], None, ps["w1"], ps["w2"], ps["w3"], top_k=K, route_norm=True)
+            if deferred:
+                with F_.defer_weight_grads() as q:
+                    out.sum().backward()
+                assert len(q) == 2 and (ps["w1"].grad is None or _ == 1)
+                q.run()
+            else:
+                out.sum().backward()
+        return {k: p.grad.clone() for k, p in ps.items()}
+
+    ref, got = run(False), run(True)
+    for k in NAMES:
+        assert rel_err(got[k], ref[k]) <= 1e-6, k
