@@ -125,10 +125,11 @@ PK_API int pk_permute_bwd(const void* d_routed, int dtype, const int32_t* inv_pe
 
 /* out[t,:] = sum_k top_scores[t,k] * y_sorted[inv_perm[t*K+k], :], fp32 accumulation in
  * ascending k, rounded once to `dtype`.  Fuses the unpermute scatter and the fp32 bmm
- * combine (qwen3.py:265-283). */
+ * combine (qwen3.py:265-283).  residual (optional, [T,H] in `dtype`) is added to the rounded
+ * sum, which fuses the block's `x + moe(...)` (qwen3.py:313-314). */
 PK_API int pk_combine_fwd(const void* y_sorted, int dtype, const int32_t* inv_perm,
-                   const float* top_scores, void* out, int64_t T, int64_t H, int64_t K,
-                   pk_stream_t stream);
+                   const float* top_scores, const void* residual, void* out, int64_t T, int64_t H,
+                   int64_t K, pk_stream_t stream);
 
 /* Backward of pk_combine_fwd, per sorted row p (slot = perm[p], t = slot / K):
  *   d_y_sorted[p,:]     = top_scores[slot] * d_out[t,:]          (dtype)
@@ -136,6 +137,24 @@ PK_API int pk_combine_fwd(const void* y_sorted, int dtype, const int32_t* inv_pe
 PK_API int pk_combine_bwd(const void* d_out, const void* y_sorted, int dtype, const int32_t* perm,
                    const float* top_scores, void* d_y_sorted, float* d_top_scores, int64_t A,
                    int64_t H, int64_t K, pk_stream_t stream);
+
+/* ------------------------------------------------------ RMSNorm in front of the region
+ * The block's ffn_norm (qwen3.py:313-314; torchtitan builds it as RMSNorm(dim, eps=norm_eps),
+ * eps 1e-6 in the Qwen3 configs, qwen3.py:28): y = x * rsqrt(mean_h(x^2) + eps) * weight, computed
+ * in fp32 and rounded once.  x, weight, y in `dtype`; rstd [T] f32 (optional) is what the
+ * backward needs. */
+PK_API int pk_rmsnorm_fwd(const void* x, int dtype, const void* weight, float eps, void* y, float* rstd,
+                   int64_t T, int64_t H, pk_stream_t stream);
+/* Backward.  d_x = rstd * (s - xh * mean_h(s * xh)) with xh = x * rstd, s = d_y * weight;
+ * d_x_addend (optional, [T,H] in `dtype`, e.g. the gradient of the residual branch) is added to
+ * the rounded result.  d_weight (optional, [H] in `dtype`) = sum_t d_y * xh, summed in a fixed
+ * order through `workspace` (pk_rmsnorm_bwd_workspace_bytes); accumulate adds to what is there.
+ * Rows of up to 8192 (bf16) / 4096 (f32) elements with 16-byte aligned operands run in one
+ * pass with d_weight partials in registers; other shapes take a slower generic pair of kernels. */
+PK_API int64_t pk_rmsnorm_bwd_workspace_bytes(int64_t T, int64_t H);
+PK_API int pk_rmsnorm_bwd(const void* d_y, const void* x, int dtype, const void* weight, const float* rstd,
+                   const void* d_x_addend, void* d_x, void* d_weight, int accumulate, int64_t T,
+                   int64_t H, void* workspace, int64_t workspace_bytes, pk_stream_t stream);
 
 /* ------------------------------------------------------ grouped SwiGLU experts
  * Expert e owns rows [starts[e], starts[e+1]) of every [A, *] operand.

@@ -17,7 +17,10 @@ Pinning status (tests/test_oracle_*.py):
                                (padded_bmm_experts below) and a per-row float64 evaluation
   unpermute_combine            float64 evaluation of sum_k s[t,k] * y[t,k,:]
   backward                     torch.autograd over this forward; gradcheck in float64
-  torchtitan op order/dtypes   PARITY UNPINNED: cannot be pinned offline (library absent)
+  rmsnorm / moe_block          library routine torch.nn.functional.rms_norm (present on CPU) and the
+                               closed form x / sqrt(mean(x^2) + eps) * w in float64; gradcheck
+  torchtitan op order/dtypes   PARITY UNPINNED: cannot be pinned offline (library absent); this
+                               covers the router, the reorderer and the block's ffn_norm module
 """
 from __future__ import annotations
 
@@ -144,3 +147,19 @@ def moe_forward(x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale
     aux = dict(logits=logits, top_scores=top_scores, top_idx=top_idx, counts=counts, starts=starts,
                perm=perm, inv_perm=inv_perm, y_sorted=y)
     return out, aux
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """The block's ffn_norm (qwen3.py:313-314; built by torchtitan as RMSNorm(dim, eps=norm_eps),
+    qwen3.py:28): x * rsqrt(mean(x^2) + eps) * weight over the last dimension, evaluated in the
+    dtype of x (float32 / float64 in the tests)."""
+    ms = x.pow(2).mean(dim=-1, keepdim=True)
+    return x * torch.rsqrt(ms + eps) * weight
+
+
+def moe_block(h, norm_weight, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale=1.0, norm_eps=1e-6,
+              compute_dtype=None):
+    """h + moe(ffn_norm(h)) (qwen3.py:313-314) on h [T,H]."""
+    out, aux = moe_forward(rmsnorm(h, norm_weight, norm_eps), w_gate, gate_bias, w1, w2, w3, top_k, route_norm,
+                           route_scale, compute_dtype=compute_dtype)
+    return h + out, aux

@@ -37,7 +37,10 @@ SIGNATURES = {
     "pk_counts_to_starts": (_c_int, [_p, _c_int, _c_i64, _p, _p]),
     "pk_permute_fwd": (_c_int, [_p, _c_int, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
     "pk_permute_bwd": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
-    "pk_combine_fwd": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_combine_fwd": (_c_int, [_p, _c_int, _p, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_rmsnorm_fwd": (_c_int, [_p, _c_int, _p, _c_f32, _p, _p, _c_i64, _c_i64, _p]),
+    "pk_rmsnorm_bwd_workspace_bytes": (_c_i64, [_c_i64, _c_i64]),
+    "pk_rmsnorm_bwd": (_c_int, [_p, _p, _c_int, _p, _p, _p, _p, _p, _c_int, _c_i64, _c_i64, _p, _c_i64, _p]),
     "pk_combine_bwd": (_c_int, [_p, _p, _c_int, _p, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
     "pk_grouped_swiglu_fwd": (_c_int, [_p, _p, _c_i64, _p, _p, _p, _p, _p, _p, _p, _p,
                                        _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),

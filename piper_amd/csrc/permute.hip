@@ -54,12 +54,12 @@ __global__ __launch_bounds__(kRowThreads) void permute_fwd_kernel(
   }
 }
 
-// out[t,:] = sum_k w[t,k] * rows[inv_perm[t*K+k], :] (+ addend[t,:]);  w == nullptr -> 1
+// out[t,:] = sum_k w[t,k] * rows[inv_perm[t*K+k], :] (+ addend[t,:]) (+ residual[t,:]);  w == nullptr -> 1
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void gather_reduce_kernel(
     const T* __restrict__ rows, const int32_t* __restrict__ inv_perm,
-    const float* __restrict__ weights, const float* __restrict__ addend, T* __restrict__ out,
-    int64_t H, int K) {
+    const float* __restrict__ weights, const float* __restrict__ addend, const T* __restrict__ residual,
+    T* __restrict__ out, int64_t H, int K) {
   using IO = RowIO<T, VEC>;
   constexpr int N = PkVec16<T>::N;
   const int64_t t = blockIdx.x;
@@ -79,6 +79,12 @@ __global__ __launch_bounds__(kRowThreads) void gather_reduce_kernel(
     if (addend) {
 #pragma unroll
       for (int i = 0; i < IO::N; ++i) acc[i] += addend[t * H + v * IO::N + i];
+    }
+    if (residual) {   // the sum is rounded to T first, like a separate add of two T tensors
+      float r[N];
+      IO::load(residual + t * H, v, r);
+#pragma unroll
+      for (int i = 0; i < IO::N; ++i) acc[i] = pk_to_float<T>(pk_from_float<T>(acc[i])) + r[i];
     }
     IO::store(out + t * H, v, acc);
   }
@@ -113,12 +119,186 @@ __global__ __launch_bounds__(kRowThreads) void combine_bwd_kernel(
   if (threadIdx.x == 0) d_scores[slot] = dot;
 }
 
+// ---- RMSNorm over rows: y = x * rsqrt(mean(x^2) + eps) * w, computed in fp32 and rounded once.
+// One block per row; the row is read twice (the second read hits the cache).
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kRowThreads) void rmsnorm_fwd_kernel(
+    const T* __restrict__ x, const T* __restrict__ w, float eps, T* __restrict__ y,
+    float* __restrict__ rstd, int64_t H) {
+  using IO = RowIO<T, VEC>;
+  constexpr int N = PkVec16<T>::N;
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  const T* row = x + t * H;
+  const int64_t nv = H / IO::N;
+  float ss = 0.f;
+  for (int64_t v = threadIdx.x; v < nv; v += kRowThreads) {
+    float f[N];
+    IO::load(row, v, f);
+#pragma unroll
+    for (int i = 0; i < IO::N; ++i) ss = fmaf(f[i], f[i], ss);
+  }
+  ss = pk_block_sum(ss, red);
+  const float rs = rsqrtf(ss / (float)H + eps);
+  if (threadIdx.x == 0 && rstd) rstd[t] = rs;
+  for (int64_t v = threadIdx.x; v < nv; v += kRowThreads) {
+    float f[N], g[N];
+    IO::load(row, v, f);
+    IO::load(w, v, g);
+#pragma unroll
+    for (int i = 0; i < IO::N; ++i) f[i] = (f[i] * rs) * g[i];
+    IO::store(y + t * H, v, f);
+  }
+}
+
+// Backward: with xh = x * rstd and s = d_y * w,
+//   d_x = rstd * (s - xh * mean(s * xh)) (+ addend),   d_w[h] = sum_t d_y[t,h] * xh[t,h].
+// Block b walks rows b, b + gridDim.x, ...; every thread keeps the d_w partial sums of the
+// columns it touches in registers and writes them to partial[b, :] at the end, so the column
+// sums are reduced in a fixed order by a second kernel.  CPT = column vectors per thread.
+template <typename T, bool VEC, int CPT>
+__global__ __launch_bounds__(kRowThreads) void rmsnorm_bwd_kernel(
+    const T* __restrict__ d_y, const T* __restrict__ x, const T* __restrict__ w,
+    const float* __restrict__ rstd, const T* __restrict__ addend, T* __restrict__ d_x,
+    float* __restrict__ partial, int64_t rows, int64_t H) {
+  using IO = RowIO<T, VEC>;
+  constexpr int N = PkVec16<T>::N;
+  __shared__ float red[16];
+  const int64_t nv = H / IO::N;
+  float dw[CPT][N];
+  float wv[CPT][N];
+#pragma unroll
+  for (int c = 0; c < CPT; ++c) {
+    const int64_t v = threadIdx.x + (int64_t)c * kRowThreads;
+#pragma unroll
+    for (int i = 0; i < N; ++i) { dw[c][i] = 0.f; wv[c][i] = 0.f; }
+    if (v < nv) IO::load(w, v, wv[c]);
+  }
+  for (int64_t t = blockIdx.x; t < rows; t += gridDim.x) {
+    const float rs = rstd[t];
+    float s[CPT][N], xh[CPT][N];
+    float dot = 0.f;
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) {
+      const int64_t v = threadIdx.x + (int64_t)c * kRowThreads;
+#pragma unroll
+      for (int i = 0; i < N; ++i) { s[c][i] = 0.f; xh[c][i] = 0.f; }
+      if (v < nv) {
+        float dy[N];
+        IO::load(d_y + t * H, v, dy);
+        IO::load(x + t * H, v, xh[c]);
+#pragma unroll
+        for (int i = 0; i < IO::N; ++i) {
+          xh[c][i] *= rs;
+          s[c][i] = dy[i] * wv[c][i];
+          dw[c][i] = fmaf(dy[i], xh[c][i], dw[c][i]);
+          dot = fmaf(s[c][i], xh[c][i], dot);
+        }
+      }
+    }
+    dot = pk_block_sum(dot, red) / (float)H;
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) {
+      const int64_t v = threadIdx.x + (int64_t)c * kRowThreads;
+      if (v < nv) {
+        float o[N];
+#pragma unroll
+        for (int i = 0; i < IO::N; ++i) o[i] = rs * (s[c][i] - xh[c][i] * dot);
+        if (addend) {   // both terms are T tensors in the unfused formulation: round, then add
+          float a[N];
+          IO::load(addend + t * H, v, a);
+#pragma unroll
+          for (int i = 0; i < IO::N; ++i) o[i] = pk_to_float<T>(pk_from_float<T>(o[i])) + a[i];
+        }
+        IO::store(d_x + t * H, v, o);
+      }
+    }
+  }
+  if (partial) {
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) {
+      const int64_t v = threadIdx.x + (int64_t)c * kRowThreads;
+      if (v < nv) {
+#pragma unroll
+        for (int i = 0; i < IO::N; ++i) partial[(int64_t)blockIdx.x * H + v * IO::N + i] = dw[c][i];
+      }
+    }
+  }
+}
+
+// d_w[h] = (accumulate ? d_w[h] : 0) + sum_b partial[b, h], b ascending
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, int nb,
+                                                                 T* __restrict__ d_w, int64_t H, int accumulate) {
+  const int64_t h = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (h >= H) return;
+  float s = 0.f;
+  for (int b = 0; b < nb; ++b) s += partial[(int64_t)b * H + h];
+  if (accumulate) s += pk_to_float<T>(d_w[h]);
+  d_w[h] = pk_from_float<T>(s);
+}
+
+// Rows too long for the register-resident kernel (or not vectorisable): d_x with strided loops,
+// one block per row, and d_w as plain column sums (one thread per column, rows in order).
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void rmsnorm_bwd_dx_generic_kernel(
+    const T* __restrict__ d_y, const T* __restrict__ x, const T* __restrict__ w,
+    const float* __restrict__ rstd, const T* __restrict__ addend, T* __restrict__ d_x, int64_t H) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  const float rs = rstd[t];
+  float dot = 0.f;
+  for (int64_t h = threadIdx.x; h < H; h += kRowThreads)
+    dot = fmaf(pk_to_float<T>(d_y[t * H + h]) * pk_to_float<T>(w[h]), pk_to_float<T>(x[t * H + h]) * rs, dot);
+  dot = pk_block_sum(dot, red) / (float)H;
+  for (int64_t h = threadIdx.x; h < H; h += kRowThreads) {
+    const float xh = pk_to_float<T>(x[t * H + h]) * rs;
+    float o = rs * (pk_to_float<T>(d_y[t * H + h]) * pk_to_float<T>(w[h]) - xh * dot);
+    if (addend) o = pk_to_float<T>(pk_from_float<T>(o)) + pk_to_float<T>(addend[t * H + h]);
+    d_x[t * H + h] = pk_from_float<T>(o);
+  }
+}
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_dw_generic_kernel(const T* __restrict__ d_y, const T* __restrict__ x,
+                                                                  const float* __restrict__ rstd, T* __restrict__ d_w,
+                                                                  int64_t rows, int64_t H, int accumulate) {
+  const int64_t h = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (h >= H) return;
+  float s = 0.f;
+  for (int64_t t = 0; t < rows; ++t) s = fmaf(pk_to_float<T>(d_y[t * H + h]), pk_to_float<T>(x[t * H + h]) * rstd[t], s);
+  if (accumulate) s += pk_to_float<T>(d_w[h]);
+  d_w[h] = pk_from_float<T>(s);
+}
+
+constexpr int kNormBwdBlocks = 512;
+constexpr int kNormBwdMaxCpt = 4;   // column vectors per thread
+
 bool vec_ok(int dtype, int64_t H, std::initializer_list<const void*> ptrs) {
   const int n = dtype == PK_BF16 ? 8 : 4;
   if (H % n != 0) return false;
   for (const void* p : ptrs)
     if (p && !pk_aligned16(p)) return false;
   return true;
+}
+
+
+template <typename T, bool VEC>
+int rmsnorm_bwd_launch(const void* d_y, const void* x, const void* weight, const float* rstd,
+                       const void* addend, void* d_x, float* partial, int64_t rows, int64_t H,
+                       int nb, hipStream_t s) {
+  const int64_t nv = H / (VEC ? PkVec16<T>::N : 1);
+  const int64_t cpt = pk_ceil_div(nv, kRowThreads);
+  const dim3 grid((unsigned)nb);
+#define PK_NORM_BWD(C)                                                                                       \
+  PK_LAUNCH_NOCHECK(pk_timing::K_RMSNORM_BWD, s, (rmsnorm_bwd_kernel<T, VEC, C>), grid, dim3(kRowThreads), 0, s, \
+                    (const T*)d_y, (const T*)x, (const T*)weight, rstd, (const T*)addend, (T*)d_x, partial, rows, H)
+  if (cpt <= 1) { PK_NORM_BWD(1); }
+  else if (cpt <= 2) { PK_NORM_BWD(2); }
+  else if (cpt <= kNormBwdMaxCpt) { PK_NORM_BWD(4); }
+  else return PK_ERR_UNSUPPORTED;   // the caller takes the generic kernels
+#undef PK_NORM_BWD
+  PK_RETURN_IF_LAUNCH_FAILED();
+  return PK_OK;
 }
 
 }  // namespace
@@ -146,21 +326,21 @@ int pk_permute_fwd(const void* x, int dtype, const int32_t* perm, void* routed, 
 }
 
 static int gather_reduce(const void* rows, int dtype, const int32_t* inv_perm, const float* weights,
-                         const float* addend, void* out, int64_t T, int64_t H, int64_t K,
-                         pk_stream_t stream) {
+                         const float* addend, const void* residual, void* out, int64_t T, int64_t H,
+                         int64_t K, pk_stream_t stream) {
   if (T < 0 || H <= 0 || K <= 0 || !pk_dtype_ok(dtype)) return PK_ERR_ARG;
   if (T == 0) return PK_OK;
   if (!rows || !inv_perm || !out) return PK_ERR_ARG;
   if (T > 0x7fffffffll) return PK_ERR_SHAPE;
-  const bool vec = vec_ok(dtype, H, {rows, out});
+  const bool vec = vec_ok(dtype, H, {rows, out, residual});
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)T);
   if (dtype == PK_BF16) {
-    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<bf16_t, true>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)rows, inv_perm, weights, addend, (bf16_t*)out, H, (int)K);
-    else PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<bf16_t, false>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)rows, inv_perm, weights, addend, (bf16_t*)out, H, (int)K);
+    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<bf16_t, true>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)rows, inv_perm, weights, addend, (const bf16_t*)residual, (bf16_t*)out, H, (int)K);
+    else PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<bf16_t, false>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)rows, inv_perm, weights, addend, (const bf16_t*)residual, (bf16_t*)out, H, (int)K);
   } else {
-    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<float, true>), grid, dim3(kRowThreads), 0, s, (const float*)rows, inv_perm, weights, addend, (float*)out, H, (int)K);
-    else PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<float, false>), grid, dim3(kRowThreads), 0, s, (const float*)rows, inv_perm, weights, addend, (float*)out, H, (int)K);
+    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<float, true>), grid, dim3(kRowThreads), 0, s, (const float*)rows, inv_perm, weights, addend, (const float*)residual, (float*)out, H, (int)K);
+    else PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<float, false>), grid, dim3(kRowThreads), 0, s, (const float*)rows, inv_perm, weights, addend, (const float*)residual, (float*)out, H, (int)K);
   }
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
@@ -169,14 +349,14 @@ static int gather_reduce(const void* rows, int dtype, const int32_t* inv_perm, c
 int pk_permute_bwd(const void* d_routed, int dtype, const int32_t* inv_perm,
                    const float* addend_f32, void* d_x, int64_t T, int64_t H, int64_t K,
                    pk_stream_t stream) {
-  return gather_reduce(d_routed, dtype, inv_perm, nullptr, addend_f32, d_x, T, H, K, stream);
+  return gather_reduce(d_routed, dtype, inv_perm, nullptr, addend_f32, nullptr, d_x, T, H, K, stream);
 }
 
 int pk_combine_fwd(const void* y_sorted, int dtype, const int32_t* inv_perm,
-                   const float* top_scores, void* out, int64_t T, int64_t H, int64_t K,
-                   pk_stream_t stream) {
+                   const float* top_scores, const void* residual, void* out, int64_t T, int64_t H,
+                   int64_t K, pk_stream_t stream) {
   if (!top_scores && T > 0) return PK_ERR_ARG;
-  return gather_reduce(y_sorted, dtype, inv_perm, top_scores, nullptr, out, T, H, K, stream);
+  return gather_reduce(y_sorted, dtype, inv_perm, top_scores, nullptr, residual, out, T, H, K, stream);
 }
 
 int pk_combine_bwd(const void* d_out, const void* y_sorted, int dtype, const int32_t* perm,
@@ -197,6 +377,78 @@ int pk_combine_bwd(const void* d_out, const void* y_sorted, int dtype, const int
     else PK_LAUNCH_NOCHECK(pk_timing::K_COMBINE_BWD, s, (combine_bwd_kernel<float, false>), grid, dim3(kRowThreads), 0, s, (const float*)d_out, (const float*)y_sorted, perm, top_scores, (float*)d_y_sorted, d_top_scores, H, (int)K);
   }
   PK_RETURN_IF_LAUNCH_FAILED();
+  return PK_OK;
+}
+
+int pk_rmsnorm_fwd(const void* x, int dtype, const void* weight, float eps, void* y, float* rstd,
+                   int64_t T, int64_t H, pk_stream_t stream) {
+  if (T < 0 || H <= 0 || !pk_dtype_ok(dtype) || !(eps >= 0.f)) return PK_ERR_ARG;
+  if (T == 0) return PK_OK;
+  if (!x || !weight || !y) return PK_ERR_ARG;
+  if (T > 0x7fffffffll) return PK_ERR_SHAPE;
+  const bool vec = vec_ok(dtype, H, {x, weight, y});
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)T);
+  if (dtype == PK_BF16) {
+    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_RMSNORM_FWD, s, (rmsnorm_fwd_kernel<bf16_t, true>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)x, (const bf16_t*)weight, eps, (bf16_t*)y, rstd, H);
+    else PK_LAUNCH_NOCHECK(pk_timing::K_RMSNORM_FWD, s, (rmsnorm_fwd_kernel<bf16_t, false>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)x, (const bf16_t*)weight, eps, (bf16_t*)y, rstd, H);
+  } else {
+    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_RMSNORM_FWD, s, (rmsnorm_fwd_kernel<float, true>), grid, dim3(kRowThreads), 0, s, (const float*)x, (const float*)weight, eps, (float*)y, rstd, H);
+    else PK_LAUNCH_NOCHECK(pk_timing::K_RMSNORM_FWD, s, (rmsnorm_fwd_kernel<float, false>), grid, dim3(kRowThreads), 0, s, (const float*)x, (const float*)weight, eps, (float*)y, rstd, H);
+  }
+  PK_RETURN_IF_LAUNCH_FAILED();
+  return PK_OK;
+}
+
+int64_t pk_rmsnorm_bwd_workspace_bytes(int64_t T, int64_t H) {
+  if (T < 0 || H <= 0) return PK_ERR_ARG;
+  const int64_t nb = T < kNormBwdBlocks ? (T > 0 ? T : 1) : kNormBwdBlocks;
+  return nb * H * (int64_t)sizeof(float);
+}
+
+int pk_rmsnorm_bwd(const void* d_y, const void* x, int dtype, const void* weight, const float* rstd,
+                   const void* d_x_addend, void* d_x, void* d_weight, int accumulate, int64_t T,
+                   int64_t H, void* workspace, int64_t workspace_bytes, pk_stream_t stream) {
+  if (T < 0 || H <= 0 || !pk_dtype_ok(dtype)) return PK_ERR_ARG;
+  if (T == 0) return PK_OK;
+  if (!d_y || !x || !weight || !rstd || !d_x) return PK_ERR_ARG;
+  if (T > 0x7fffffffll) return PK_ERR_SHAPE;
+  const int nb = (int)(T < kNormBwdBlocks ? T : kNormBwdBlocks);
+  float* partial = nullptr;
+  if (d_weight) {
+    if (!workspace || workspace_bytes < pk_rmsnorm_bwd_workspace_bytes(T, H)) return PK_ERR_WORKSPACE;
+    partial = reinterpret_cast<float*>(workspace);
+  }
+  const bool vec = vec_ok(dtype, H, {d_y, x, weight, d_x, d_x_addend});
+  hipStream_t s = (hipStream_t)stream;
+  int rc;
+  if (dtype == PK_BF16)
+    rc = vec ? rmsnorm_bwd_launch<bf16_t, true>(d_y, x, weight, rstd, d_x_addend, d_x, partial, T, H, nb, s)
+             : rmsnorm_bwd_launch<bf16_t, false>(d_y, x, weight, rstd, d_x_addend, d_x, partial, T, H, nb, s);
+  else
+    rc = vec ? rmsnorm_bwd_launch<float, true>(d_y, x, weight, rstd, d_x_addend, d_x, partial, T, H, nb, s)
+             : rmsnorm_bwd_launch<float, false>(d_y, x, weight, rstd, d_x_addend, d_x, partial, T, H, nb, s);
+  if (rc == PK_ERR_UNSUPPORTED) {
+    const dim3 rows_grid((unsigned)T), cols_grid((unsigned)pk_ceil_div(H, 256));
+    if (dtype == PK_BF16) {
+      PK_LAUNCH_NOCHECK(pk_timing::K_RMSNORM_BWD, s, (rmsnorm_bwd_dx_generic_kernel<bf16_t>), rows_grid, dim3(kRowThreads), 0, s, (const bf16_t*)d_y, (const bf16_t*)x, (const bf16_t*)weight, rstd, (const bf16_t*)d_x_addend, (bf16_t*)d_x, H);
+      if (d_weight) PK_LAUNCH_NOCHECK(pk_timing::K_RMSNORM_BWD, s, (rmsnorm_dw_generic_kernel<bf16_t>), cols_grid, dim3(256), 0, s, (const bf16_t*)d_y, (const bf16_t*)x, rstd, (bf16_t*)d_weight, T, H, accumulate ? 1 : 0);
+    } else {
+      PK_LAUNCH_NOCHECK(pk_timing::K_RMSNORM_BWD, s, (rmsnorm_bwd_dx_generic_kernel<float>), rows_grid, dim3(kRowThreads), 0, s, (const float*)d_y, (const float*)x, (const float*)weight, rstd, (const float*)d_x_addend, (float*)d_x, H);
+      if (d_weight) PK_LAUNCH_NOCHECK(pk_timing::K_RMSNORM_BWD, s, (rmsnorm_dw_generic_kernel<float>), cols_grid, dim3(256), 0, s, (const float*)d_y, (const float*)x, rstd, (float*)d_weight, T, H, accumulate ? 1 : 0);
+    }
+    PK_RETURN_IF_LAUNCH_FAILED();
+    return PK_OK;
+  }
+  if (rc != PK_OK) return rc;
+  if (d_weight) {
+    const dim3 grid((unsigned)pk_ceil_div(H, 256));
+    if (dtype == PK_BF16)
+      PK_LAUNCH_NOCHECK(pk_timing::K_RMSNORM_BWD, s, (rmsnorm_dw_reduce_kernel<bf16_t>), grid, dim3(256), 0, s, partial, nb, (bf16_t*)d_weight, H, accumulate ? 1 : 0);
+    else
+      PK_LAUNCH_NOCHECK(pk_timing::K_RMSNORM_BWD, s, (rmsnorm_dw_reduce_kernel<float>), grid, dim3(256), 0, s, partial, nb, (float*)d_weight, H, accumulate ? 1 : 0);
+    PK_RETURN_IF_LAUNCH_FAILED();
+  }
   return PK_OK;
 }
 

@@ -269,13 +269,13 @@ class _ExpertRegionFn(torch.autograd.Function):
     """x [T,H] -> out [T,H]; saves the routing tables and the SwiGLU pre-activations."""
 
     @staticmethod
-    def forward(ctx, x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale):
+    def forward(ctx, x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale, residual=None):
         E = w1.shape[0]
         logits = ops.gate_logits(x, w_gate, gate_bias)
         top_scores, top_idx = ops.route_topk(logits, top_k, route_norm, route_scale)
         _counts, starts, perm, inv_perm, order = ops.sort_by_expert(top_idx, E, with_order=True)
         y, g, u, h = ops.grouped_swiglu_fwd(x, w1, w2, w3, starts, row_map=perm, row_map_div=top_k)
-        out = ops.combine_fwd(y, inv_perm, top_scores)
+        out = ops.combine_fwd(y, inv_perm, top_scores, residual)
         ctx.save_for_backward(x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, h, y, order)
         ctx.cfg = (top_k, route_norm, route_scale, gate_bias is not None)
         ctx.params = (w_gate, gate_bias, w1, w2, w3)
@@ -319,7 +319,7 @@ class _ExpertRegionFn(torch.autograd.Function):
                     p_bias.grad = gb
 
             _WGRAD_QUEUE.push(run_router)
-            return d_x, None, None, None, None, None, None, None, None
+            return d_x, None, None, None, None, None, None, None, None, (d_out if need[9] else None)
         side = _side_stream(x.device) if (need[3] or need[4] or need[5]) and _OVERLAP_WGRAD else None
         if need[3] or need[4] or need[5]:
             if side is not None:
@@ -340,9 +340,39 @@ class _ExpertRegionFn(torch.autograd.Function):
                 t.record_stream(side)
             for t in (d_w1, d_w2, d_w3):     # allocated on the side stream, consumed on the current one
                 t.record_stream(cur)
-        return d_x, d_wg, d_b, d_w1, d_w2, d_w3, None, None, None
+        return d_x, d_wg, d_b, d_w1, d_w2, d_w3, None, None, None, (d_out if need[9] else None)
 
 
-def expert_region(x, w_gate, gate_bias, w1, w2, w3, *, top_k: int, route_norm: bool, route_scale: float = 1.0):
-    """The whole MoE expert region of AnnotatedMoE.forward (qwen3.py:233-289) on x [T,H]."""
-    return _ExpertRegionFn.apply(x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale)
+def expert_region(x, w_gate, gate_bias, w1, w2, w3, *, top_k: int, route_norm: bool, route_scale: float = 1.0,
+                  residual=None):
+    """The whole MoE expert region of AnnotatedMoE.forward (qwen3.py:233-289) on x [T,H].
+    `residual` [T,H] is added to the result in the combine kernel."""
+    return _ExpertRegionFn.apply(x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale, residual)
+
+
+class _RMSNormFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, eps):
+        y, rstd = ops.rmsnorm_fwd(x, weight, eps)
+        ctx.save_for_backward(x, weight, rstd)
+        return y
+
+    @staticmethod
+    def backward(ctx, d_y):
+        x, weight, rstd = ctx.saved_tensors
+        d_x, d_w = ops.rmsnorm_bwd(d_y, x, weight, rstd, need_dw=ctx.needs_input_grad[1])
+        return (d_x if ctx.needs_input_grad[0] else None), d_w, None
+
+
+def rmsnorm(x, weight, eps: float = 1e-6):
+    """RMSNorm over the last dimension (the block's ffn_norm, qwen3.py:313-314)."""
+    shape = x.shape
+    return _RMSNormFn.apply(x.reshape(-1, shape[-1]), weight, eps).reshape(shape)
+
+
+def moe_block(h, norm_weight, w_gate, gate_bias, w1, w2, w3, *, top_k: int, route_norm: bool,
+              route_scale: float = 1.0, norm_eps: float = 1e-6):
+    """h + moe(ffn_norm(h)) on h [T,H] (qwen3.py:313-314): RMSNorm kernel, expert region, residual
+    added in the combine kernel."""
+    return expert_region(rmsnorm(h, norm_weight, norm_eps), w_gate, gate_bias, w1, w2, w3, top_k=top_k,
+                         route_norm=route_norm, route_scale=route_scale, residual=h)

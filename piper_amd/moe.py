@@ -104,7 +104,8 @@ class AnnotatedMoE(nn.Module):
         if self.router.gate.bias is not None:
             nn.init.zeros_(self.router.gate.bias)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, residual: torch.Tensor | None = None) -> torch.Tensor:
+        """``residual`` (same shape as x; fused path only) is added in the combine kernel."""
         bs, slen, dim = x.shape
         x2 = x.reshape(-1, dim)
         top_k = self.router.top_k
@@ -112,8 +113,11 @@ class AnnotatedMoE(nn.Module):
             with annotate(EP_TAG):
                 out = F_.expert_region(x2, self.router.gate.weight, self.router.gate.bias, self.experts.w1,
                                        self.experts.w2, self.experts.w3, top_k=top_k,
-                                       route_norm=self.router.route_norm, route_scale=self.router.route_scale)
+                                       route_norm=self.router.route_norm, route_scale=self.router.route_scale,
+                                       residual=None if residual is None else residual.reshape(-1, dim))
             return out.reshape(bs, slen, dim)
+        if residual is not None:
+            return residual + self.forward(x)
 
         top_scores, selected_experts_indices, num_tokens_per_expert = self.router(x2, self.expert_bias)
         _scores_sorted, token_indices_experts_sorted, num_tokens_per_expert = self.reorderer(
@@ -123,3 +127,30 @@ class AnnotatedMoE(nn.Module):
             gathered_output = self.experts(routed_input, num_tokens_per_expert)
         out_experts = F_.combine(gathered_output.reshape(-1, dim), token_indices_experts_sorted, top_scores)
         return out_experts.reshape(bs, slen, dim)
+
+
+class RMSNorm(nn.Module):
+    """The norm module torchtitan's TransformerBlock builds as ``ffn_norm`` (RMSNorm(dim, eps))."""
+
+    def __init__(self, dim: int, eps: float = 1e-6, dtype: torch.dtype | None = None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim, dtype=dtype))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return F_.rmsnorm(x, self.weight, self.eps)
+
+
+class MoEFeedForwardBlock(nn.Module):
+    """The MoE half of AnnotatedQwen3TransformerBlock.forward (qwen3.py:313-314):
+    ``x = x + self.moe(self.ffn_norm(x))`` with the parameter names of the reference block
+    (``ffn_norm.weight``, ``moe.router.gate.weight``, ``moe.experts.w1/w2/w3``)."""
+
+    def __init__(self, moe_args: MoEArgs, dim: int, hidden_dim: int, norm_eps: float = 1e-6,
+                 dtype: torch.dtype | None = None):
+        super().__init__()
+        self.ffn_norm = RMSNorm(dim, norm_eps, dtype=dtype)
+        self.moe = AnnotatedMoE(moe_args, dim, hidden_dim, dtype=dtype, fused=True)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.moe(self.ffn_norm(x), residual=x)

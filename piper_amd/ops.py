@@ -139,16 +139,56 @@ def permute_bwd(d_routed: torch.Tensor, inv_perm: torch.Tensor, top_k: int, adde
     return d_x
 
 
-def combine_fwd(y_sorted: torch.Tensor, inv_perm: torch.Tensor, top_scores: torch.Tensor) -> torch.Tensor:
+def combine_fwd(y_sorted: torch.Tensor, inv_perm: torch.Tensor, top_scores: torch.Tensor,
+                residual: torch.Tensor | None = None) -> torch.Tensor:
+    """Unpermute + weighted combine; `residual` [T,H] (same dtype) is added to the rounded sum."""
     require_gpu(y_sorted)
     A, H = y_sorted.shape
     T, K = top_scores.shape
     _check(A == T * K, "combine_fwd: y_sorted rows must equal T*K")
     y_sorted = y_sorted.contiguous()
+    if residual is not None:
+        _check(residual.shape == (T, H) and residual.dtype == y_sorted.dtype, "combine_fwd: residual must be [T,H] in the dtype of y")
+        residual = residual.contiguous()
     out = torch.empty((T, H), dtype=y_sorted.dtype, device=y_sorted.device)
     call("pk_combine_fwd", ptr(y_sorted), dtype_code(y_sorted.dtype), ptr(inv_perm), ptr(top_scores.contiguous()),
-         ptr(out), T, H, K, current_stream(y_sorted.device))
+         ptr(residual), ptr(out), T, H, K, current_stream(y_sorted.device))
     return out
+
+
+def rmsnorm_fwd(x: torch.Tensor, weight: torch.Tensor, eps: float):
+    """y = x * rsqrt(mean(x^2) + eps) * weight over the last dimension of x [T,H].  Returns (y, rstd f32 [T])."""
+    require_gpu(x)
+    _check(x.dim() == 2 and weight.shape == (x.shape[1],) and weight.dtype == x.dtype, "rmsnorm_fwd: x [T,H], weight [H] in the dtype of x")
+    T, H = x.shape
+    x = x.contiguous()
+    y = torch.empty_like(x)
+    rstd = torch.empty(T, dtype=torch.float32, device=x.device)
+    call("pk_rmsnorm_fwd", ptr(x), dtype_code(x.dtype), ptr(weight.contiguous()), float(eps), ptr(y), ptr(rstd), T, H,
+         current_stream(x.device))
+    return y, rstd
+
+
+def rmsnorm_bwd(d_y: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: torch.Tensor, *,
+                d_x_addend: torch.Tensor | None = None, need_dw: bool = True, d_weight: torch.Tensor | None = None,
+                accumulate: bool = False):
+    """Returns (d_x, d_weight or None); d_x_addend is added to d_x in the same pass."""
+    require_gpu(d_y)
+    T, H = x.shape
+    d_y, x = d_y.contiguous(), x.contiguous()
+    d_x = torch.empty_like(x)
+    ws = None
+    if need_dw:
+        if d_weight is None:
+            _check(not accumulate, "rmsnorm_bwd: accumulate needs d_weight")
+            d_weight = torch.empty_like(weight)
+        ws = torch.empty(int(_lib.load().pk_rmsnorm_bwd_workspace_bytes(T, H)), dtype=torch.uint8, device=x.device)
+    else:
+        d_weight = None
+    call("pk_rmsnorm_bwd", ptr(d_y), ptr(x), dtype_code(x.dtype), ptr(weight.contiguous()), ptr(rstd),
+         ptr(None if d_x_addend is None else d_x_addend.contiguous()), ptr(d_x), ptr(d_weight), int(bool(accumulate)),
+         T, H, ptr(ws), 0 if ws is None else ws.numel(), current_stream(x.device))
+    return d_x, d_weight
 
 
 def combine_bwd(d_out: torch.Tensor, y_sorted: torch.Tensor, perm: torch.Tensor, top_scores: torch.Tensor):

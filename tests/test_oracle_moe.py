@@ -173,3 +173,25 @@ def test_backward_gradcheck_float64_with_empty_expert():
     for a, b in zip(g32, g64):
         assert torch.allclose(a.double(), b, atol=1e-4, rtol=1e-3)
     assert float(g64[2][2].abs().max()) == 0.0  # the empty expert gets an exactly zero weight gradient
+
+
+def test_rmsnorm_matches_library_routine_and_closed_form():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(7, 48, generator=g, dtype=torch.float64)
+    w = torch.randn(48, generator=g, dtype=torch.float64)
+    for eps in (1e-6, 1e-5, 0.5):
+        got = O.rmsnorm(x, w, eps)
+        assert torch.allclose(got, torch.nn.functional.rms_norm(x, (48,), w, eps), rtol=1e-12, atol=1e-12)
+        # closed form, element by element
+        for t in (0, 3, 6):
+            ms = sum(float(v) ** 2 for v in x[t]) / 48
+            ref = [float(x[t, h]) / (ms + eps) ** 0.5 * float(w[h]) for h in range(48)]
+            assert max(abs(float(got[t, h]) - ref[h]) for h in range(48)) < 1e-12
+    # scale invariance (up to eps): rmsnorm(c*x) == rmsnorm(x) for eps -> 0
+    assert torch.allclose(O.rmsnorm(3.0 * x, w, 0.0), O.rmsnorm(x, w, 0.0), rtol=1e-12, atol=1e-12)
+    # a row of ones with unit weight has unit RMS
+    one = torch.ones(1, 48, dtype=torch.float64)
+    assert torch.allclose(O.rmsnorm(one, torch.ones(48, dtype=torch.float64), 0.0), one)
+    xr = x.clone().requires_grad_(True)
+    wr = w.clone().requires_grad_(True)
+    assert torch.autograd.gradcheck(lambda a, b: O.rmsnorm(a, b, 1e-6), (xr, wr), eps=1e-6, atol=1e-6)
