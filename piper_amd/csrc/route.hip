@@ -173,19 +173,36 @@ __global__ __launch_bounds__(1024) void sort_scan_kernel(int32_t* __restrict__ c
                                                          int32_t* __restrict__ counts,
                                                          int32_t* __restrict__ starts,
                                                          int32_t* __restrict__ order) {
+  // One block.  The 1024 threads form G = 1024 / Epad groups (Epad = E rounded up to a power of
+  // two); group g of expert e walks chunks [g*cpg, (g+1)*cpg), so the two passes over the
+  // chunk histograms are G times shorter than with one thread per expert.
+  __shared__ int32_t part[1024];     // [g][e]: rows of expert e in the chunks of group g
   __shared__ int32_t scan[PK_MAX_EXPERTS];
   __shared__ int32_t cnts[PK_MAX_EXPERTS];
-  const int e = threadIdx.x;
-  int total = 0;
-  if (e < E) {
-    // pass 1 only reads (the loads pipeline), pass 2 rewrites each entry with its prefix
-    for (int c = 0; c < nchunks; ++c) total += chunk_hist[(int64_t)c * E + e];
-    if (counts) counts[e] = total;
-  }
-  scan[e] = (e < E) ? total : 0;
-  cnts[e] = (e < E) ? total : -1;
+  int epad = 1;
+  while (epad < E) epad <<= 1;
+  const int G = 1024 / epad;
+  const int e = threadIdx.x % epad, g = threadIdx.x / epad;
+  const int cpg = (nchunks + G - 1) / G;
+  const int c0 = g * cpg, c1 = min(nchunks, c0 + cpg);
+  int mine = 0;
+  if (e < E)
+    for (int c = c0; c < c1; ++c) mine += chunk_hist[(int64_t)c * E + e];
+  part[threadIdx.x] = mine;
   __syncthreads();
-  if (order && e < E) {
+  int total = 0, before = 0;      // rows of expert e in all chunks / in the chunks of earlier groups
+  for (int k = 0; k < G; ++k) {
+    const int v = part[k * epad + e];
+    total += v;
+    before += k < g ? v : 0;
+  }
+  if (threadIdx.x < 1024 && g == 0) {
+    if (e < E && counts) counts[e] = total;
+    scan[e] = (e < E) ? total : 0;
+    cnts[e] = (e < E) ? total : -1;
+  }
+  __syncthreads();
+  if (order && g == 0 && e < E) {
     // experts by descending row count, ties by index: order[rank] = e
     int rank = 0;
     for (int o = 0; o < E; ++o) {
@@ -194,19 +211,22 @@ __global__ __launch_bounds__(1024) void sort_scan_kernel(int32_t* __restrict__ c
     }
     order[rank] = e;
   }
-  // Hillis-Steele inclusive scan over 1024 entries
-  for (int off = 1; off < 1024; off <<= 1) {
-    const int v = (e >= off) ? scan[e - off] : 0;
+  // Hillis-Steele inclusive scan over the Epad expert totals
+  for (int off = 1; off < epad; off <<= 1) {
+    int v = 0;
+    if (g == 0 && e >= off) v = scan[e - off];
     __syncthreads();
-    scan[e] += v;
+    if (g == 0) scan[e] += v;
     __syncthreads();
   }
   const int start = scan[e] - total;  // exclusive
   if (e < E) {
-    starts[e] = start;
-    if (e == E - 1) starts[E] = scan[e];
-    int run = start;
-    for (int c = 0; c < nchunks; ++c) {
+    if (g == 0) {
+      starts[e] = start;
+      if (e == E - 1) starts[E] = scan[e];
+    }
+    int run = start + before;
+    for (int c = c0; c < c1; ++c) {
       const int v = chunk_hist[(int64_t)c * E + e];
       chunk_hist[(int64_t)c * E + e] = run;
       run += v;
