@@ -105,6 +105,7 @@ def bench_region(cfg, steps: int, warmup: int):
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
+    enqueue = time.perf_counter() - t0      # host time to launch everything (the GPU runs behind it)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     records = _lib.timing_collect()
@@ -116,6 +117,7 @@ def bench_region(cfg, steps: int, warmup: int):
         per_kernel[name] = (tot + ms, n + 1)
     summary = {k: {"launches_per_step": n / steps, "avg_ms": tot / n, "ms_per_step": tot / steps}
                for k, (tot, n) in per_kernel.items()}
+    summary["__host_enqueue_s"] = enqueue
     return elapsed, summary
 
 
@@ -238,6 +240,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     elapsed, kernels = bench_region(cfg, args.steps, args.warmup)
+    host_enqueue = kernels.pop("__host_enqueue_s")
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = cfg.tokens * args.steps / elapsed
     gemm_flops_step = cfg.gemm_flops_per_token * cfg.tokens
@@ -280,6 +283,7 @@ def main():
         "config": {"workload": f"{cfg.name}: T={cfg.tokens} H={cfg.hidden} E={cfg.num_experts} top{cfg.top_k} "
                                f"I={cfg.inter}, bf16 experts, fp32 router, fwd+bwd incl. router and all expert weight grads",
                    "tokens_per_step": cfg.tokens},
+        "host_enqueue_ms_per_step": host_enqueue / args.steps * 1e3,
         "mfma_frac_of_peak_region": mfma_frac_region,
         "gemm_tflops_region": gemm_flops_step / (ms_per_step * 1e-3) / 1e12,
         "roofline": roof,
