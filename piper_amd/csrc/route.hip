@@ -1,6 +1,6 @@
 // Routing: gate logits, wavefront softmax/top-k (+ backward), stable counting sort by expert.
 #include "pk_common.h"
-#include "mfma_f32_gemm.h"
+#include "mfma_x3_gemm.h"
 
 namespace {
 
@@ -355,12 +355,12 @@ int pk_gate_logits(const void* x, int x_dtype, const float* w_gate, const float*
   int rc;
   if (E > 64) {  // 64-token x 128-expert tiles, 8 waves
     rc = x_dtype == PK_BF16
-             ? pk_f32mm::launch<2, 4, true, true, bf16_t, float>(p, pk_timing::K_GATE_LOGITS, s)
-             : pk_f32mm::launch<2, 4, true, true, float, float>(p, pk_timing::K_GATE_LOGITS, s);
+             ? pk_x3mm::launch<2, 4, true, true, bf16_t, float>(p, pk_timing::K_GATE_LOGITS, s)
+             : pk_x3mm::launch<2, 4, true, true, float, float>(p, pk_timing::K_GATE_LOGITS, s);
   } else {       // 64-token x 64-expert tiles, 4 waves
     rc = x_dtype == PK_BF16
-             ? pk_f32mm::launch<2, 2, true, true, bf16_t, float>(p, pk_timing::K_GATE_LOGITS, s)
-             : pk_f32mm::launch<2, 2, true, true, float, float>(p, pk_timing::K_GATE_LOGITS, s);
+             ? pk_x3mm::launch<2, 2, true, true, bf16_t, float>(p, pk_timing::K_GATE_LOGITS, s)
+             : pk_x3mm::launch<2, 2, true, true, float, float>(p, pk_timing::K_GATE_LOGITS, s);
   }
   if (rc != PK_OK) return rc;
   if (sp > 1) {
@@ -398,7 +398,7 @@ int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const 
     p.M = T; p.N = H; p.K = E;
     p.sam = E; p.sak = 1; p.sbk = H; p.sbn = 1;
     p.splits = 1; p.accumulate = 0;
-    int rc = pk_f32mm::launch<2, 2, true, false, float, float>(p, pk_timing::K_GATE_LOGITS_BWD, s);
+    int rc = pk_x3mm::launch<2, 2, true, false, float, float>(p, pk_timing::K_GATE_LOGITS_BWD, s);
     if (rc != PK_OK) return rc;
   }
   if (d_w_gate) {
@@ -412,8 +412,8 @@ int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const 
     p.sam = 1; p.sak = E; p.sbk = H; p.sbn = 1;
     p.splits = sp; p.accumulate = (sp == 1 && accumulate) ? 1 : 0;
     int rc = x_dtype == PK_BF16
-                 ? pk_f32mm::launch<2, 2, false, false, float, bf16_t>(p, pk_timing::K_GATE_LOGITS_BWD, s)
-                 : pk_f32mm::launch<2, 2, false, false, float, float>(p, pk_timing::K_GATE_LOGITS_BWD, s);
+                 ? pk_x3mm::launch<2, 2, false, false, float, bf16_t>(p, pk_timing::K_GATE_LOGITS_BWD, s)
+                 : pk_x3mm::launch<2, 2, false, false, float, float>(p, pk_timing::K_GATE_LOGITS_BWD, s);
     if (rc != PK_OK) return rc;
     if (sp > 1) {
       const int64_t n = E * H;
