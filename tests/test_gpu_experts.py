@@ -144,3 +144,41 @@ def test_argument_errors(dev):
         ops.grouped_swiglu_fwd(z, w, w, w, starts)             # w2 has the wrong shape
     with pytest.raises(ValueError):
         ops.grouped_swiglu_fwd(z.float(), w, w2, w, starts)    # dtype mismatch
+
+
+def test_grouped_gemms_replay_in_a_hip_graph(dev):
+    """The persistent kernels take their work units from counters that the last workgroup of a
+    launch resets: a captured graph must give the eager result on every replay, also with new
+    input values and with eager launches in between."""
+    counts = [300, 0, 513, 77, 128, 1, 260, 5]
+    H, I = 256, 256
+    x, w1, w2, w3, dy, cnt = _make(7, counts, H, I, torch.bfloat16)
+    X, W1, W2, W3, DY = (t.to(dev) for t in (x, w1, w2, w3, dy))
+    starts = ops.counts_to_starts(cnt.to(dev))
+    E = len(counts)
+
+    def run(xin, dyin):
+        y, g, u, h = ops.grouped_swiglu_fwd(xin, W1, W2, W3, starts)
+        dx, dg, du = ops.grouped_swiglu_dgrad(dyin, W1, W2, W3, g, u, starts)
+        dw1, dw2, dw3 = ops.grouped_swiglu_wgrad(dyin, h, dg, du, xin, starts, E)
+        return y, dx, dw1, dw2, dw3
+
+    xs, dys = X.clone(), DY.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(xs, dys)                       # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = run(xs, dys)
+    for rep in range(4):
+        scale = 1.0 + 0.25 * rep
+        xs.copy_(X * scale)
+        dys.copy_(DY * (2.0 - 0.25 * rep))
+        graph.replay()
+        torch.cuda.synchronize()
+        want = run(xs.clone(), dys.clone())            # eager, between the replays
+        torch.cuda.synchronize()
+        for got, ref, name in zip(outs, want, ("y", "dx", "dw1", "dw2", "dw3")):
+            assert torch.equal(got, ref), f"replay {rep}: {name}"
