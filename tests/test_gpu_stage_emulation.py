@@ -1,0 +1,199 @@
+"""One-GPU pipeline-stage emulation (benchmark configuration 5): two Qwen3-MoE decoder layers as
+two compute buckets, microbatches in 1F1B order, parameters unflattened from a ZeRO-3-style local
+bucket before each forward, gradient packing on a second stream, one fused AdamW step.
+
+The MoE half of each layer (ffn_norm, router, experts, combine + residual) runs on the HIP kernels;
+attention (GQA with q/k RMSNorm and RoPE) is outside the accelerated path and uses torch operators
+on both sides.  A reduced shape is compared with the CPU oracle running the same layers in fp32;
+the full shape (hidden 2048, 32/4 heads of 128, 128 experts top-8, intermediate 768, 4 microbatches
+of 2 x 2048 tokens) is checked through size-independent properties."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as TF
+
+from conftest import ADAMW_TOL, BF16_TOL, rel_err
+from oracle import bucket as OB
+from oracle import moe as O
+from piper_amd import functional as F_
+from piper_amd.bucket import BucketState, ParamStorage, StageStore, flatten_params
+from piper_amd.configs import ADAMW
+from piper_amd.executor import StageExecutor, one_f_one_b
+from piper_amd.optim import FusedAdamW
+
+pytestmark = pytest.mark.gpu
+
+LAYER_PARAMS = ("attention_norm", "wq", "wk", "wv", "wo", "q_norm", "k_norm", "ffn_norm", "w1", "w3", "w2", "w_gate")
+
+
+def _layer_shapes(dim, n_heads, n_kv, hd, E, I):
+    return dict(attention_norm=(dim,), wq=(n_heads * hd, dim), wk=(n_kv * hd, dim), wv=(n_kv * hd, dim),
+                wo=(dim, n_heads * hd), q_norm=(hd,), k_norm=(hd,), ffn_norm=(dim,),
+                w1=(E, I, dim), w3=(E, I, dim), w2=(E, dim, I), w_gate=(E, dim))
+
+
+def _init_layer(gen, shapes, dtype):
+    out = {}
+    for k, s in shapes.items():
+        if k.endswith("norm"):
+            out[k] = (1.0 + 0.05 * torch.randn(s, generator=gen)).to(dtype)
+        elif k == "w_gate":
+            out[k] = torch.randn(s, generator=gen) * 0.02          # fp32 router
+        else:
+            out[k] = (torch.randn(s, generator=gen) * 0.02).to(dtype)
+    return out
+
+
+def _rope(x, theta=1e6):
+    # x [B, S, heads, hd]; rotate-half formulation
+    B, S, Hh, hd = x.shape
+    pos = torch.arange(S, device=x.device, dtype=torch.float32)
+    inv = theta ** (-torch.arange(0, hd, 2, device=x.device, dtype=torch.float32) / hd)
+    ang = pos[:, None] * inv[None, :]
+    cos, sin = ang.cos()[None, :, None, :], ang.sin()[None, :, None, :]
+    x1, x2 = x.float()[..., : hd // 2], x.float()[..., hd // 2:]
+    return torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).to(x.dtype)
+
+
+def _layer_forward(x, p, cfg, hip: bool):
+    """x [B,S,dim] -> [B,S,dim].  hip=True: RMSNorms and the MoE block on the HIP kernels."""
+    dim, n_heads, n_kv, hd, E, I, K = cfg
+    B, S, _ = x.shape
+    norm = (lambda t, w: F_.rmsnorm(t, w, 1e-6)) if hip else (lambda t, w: O.rmsnorm(t, w, 1e-6))
+    h = norm(x, p["attention_norm"])
+    q = (h @ p["wq"].t()).view(B, S, n_heads, hd)
+    k = (h @ p["wk"].t()).view(B, S, n_kv, hd)
+    v = (h @ p["wv"].t()).view(B, S, n_kv, hd)
+    q, k = _rope(norm(q, p["q_norm"])), _rope(norm(k, p["k_norm"]))
+    a = TF.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True,
+                                        enable_gqa=True)
+    x = x + a.transpose(1, 2).reshape(B, S, n_heads * hd) @ p["wo"].t()
+    x2 = x.reshape(-1, dim)
+    if hip:
+        y = F_.moe_block(x2, p["ffn_norm"], p["w_gate"], None, p["w1"], p["w2"], p["w3"], top_k=K, route_norm=True)
+    else:
+        y, _ = O.moe_block(x2, p["ffn_norm"], p["w_gate"], None, p["w1"], p["w2"], p["w3"], K, True,
+                           compute_dtype=torch.float32)
+    return y.reshape(B, S, dim)
+
+
+def _build(layers, cfg, dev, dtype):
+    """Two compute buckets (one per layer) holding the bf16 parameters, plus one fp32 bucket per
+    layer for the router gate, all ZeRO-3 style (parameters re-pointed at the bucket before use)."""
+    store = StageStore()
+    opt = lambda ps: FusedAdamW(ps, **ADAMW)
+    names = [n for n in LAYER_PARAMS if n != "w_gate"]
+    for ubid, l in enumerate(layers):
+        b = BucketState()
+        plist = {n: torch.nn.Parameter(l[n].to(dev)) for n in LAYER_PARAMS}
+        b.forward_args = [None] + [plist[n] for n in LAYER_PARAMS]
+        b.input_idxs = [0]
+        b.param_idxs = list(range(1, 1 + len(LAYER_PARAMS)))
+        b.trainable_param_idxs = list(b.param_idxs)
+        b.param_names = list(LAYER_PARAMS)
+
+        def fwd(args, _names=LAYER_PARAMS):
+            return _layer_forward(args[0], dict(zip(_names, args[1:])), cfg, True)
+
+        b.forward_fn = fwd
+        flatten_params(b, [plist[n] for n in names], optim_class=opt)
+        store.buckets[ubid] = b
+        store.zero_managed_ubids.add(ubid)
+        store.param_sharded_ubids.add(ubid)
+        gb = BucketState()
+        flatten_params(gb, [plist["w_gate"]], optim_class=opt)
+        store.buckets[f"gate{ubid}"] = gb
+        store.zero_managed_ubids.add(f"gate{ubid}")
+    compute = [0, 1]
+    view = StageStore(buckets={u: store.buckets[u] for u in compute}, zero_managed_ubids=set(compute),
+                      param_sharded_ubids=set(compute))
+    ex = StageExecutor(view, compute_stream=torch.cuda.Stream(), pack_stream=torch.cuda.Stream())
+    ex.params = ParamStorage(store)
+    orig = ex.params.accumulate_zero_param_grads_to_flat
+
+    def acc(ubid, stream=None):      # the gate bucket of a layer is packed with the layer's own bucket
+        orig(ubid, stream)
+        if f"gate{ubid}" in store.buckets:
+            orig(f"gate{ubid}", stream)
+    ex.params.accumulate_zero_param_grads_to_flat = acc
+    return store, ex, names
+
+
+def test_reduced_stage_against_cpu_oracle(dev):
+    cfg = (256, 4, 2, 64, 8, 128, 2)            # dim, heads, kv heads, head_dim, E, I, K
+    B, S, MB = 2, 64, 3
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(21)
+    shapes = _layer_shapes(*cfg[:6])
+    layers = [_init_layer(gen, shapes, dtype) for _ in range(2)]
+    xs = [torch.randn(B, S, cfg[0], generator=gen).to(dtype) for _ in range(MB)]
+
+    ref = [{k: v.clone().float().requires_grad_(True) for k, v in l.items()} for l in layers]
+    ref_losses = []
+    for x in xs:
+        h = x.float()
+        for p in ref:
+            h = _layer_forward(h, p, cfg, False)
+        loss = h.sum()
+        loss.backward()
+        ref_losses.append(loss.detach())
+
+    store, ex, names = _build(layers, cfg, dev, dtype)
+    out = ex.run(one_f_one_b(MB, [0, 1]), [x.to(dev) for x in xs])
+    torch.cuda.synchronize()
+    for got, want in zip(out["losses"], ref_losses):
+        assert abs(got.item() - want.item()) <= max(4 * BF16_TOL * abs(want.item()), 2.0)
+    # End to end the bf16 stage feeds its routers activations that differ from the fp32 oracle's by
+    # bf16 rounding (attention, previous layer), so a few near-tie tokens choose another expert and
+    # their contribution moves between expert gradients: the bound on the normalised maximum error
+    # is wide here; the per-kernel 2e-2 parity is tested on identical inputs in the other test files.
+    for ubid in (0, 1):
+        b = store.buckets[ubid]
+        for (p, off, n, shape), name in zip(b.param_view_specs, names):
+            got = b.flat_grads[off:off + n].view(shape)
+            assert rel_err(got, ref[ubid][name].grad) <= 0.25, (ubid, name)
+        gb = store.buckets[f"gate{ubid}"]
+        got = gb.flat_grads[: math.prod(shapes["w_gate"])].view(shapes["w_gate"])
+        assert rel_err(got, ref[ubid]["w_gate"].grad) <= 0.3
+
+
+def test_full_size_stage_properties(dev):
+    cfg = (2048, 32, 4, 128, 128, 768, 8)
+    B, S, MB = 2, 2048, 4
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(5)
+    shapes = _layer_shapes(*cfg[:6])
+    layers = [_init_layer(gen, shapes, dtype) for _ in range(2)]
+    vocab = 151936
+    emb = (torch.randn(4096, cfg[0], generator=gen) * 0.5).to(dtype).to(dev)     # rows of a stand-in embedding table
+    ids = [torch.randint(0, vocab, (B, S), generator=gen) for _ in range(MB)]
+    xs = [emb[(i % 4096).to(dev)] for i in ids]
+
+    store, ex, names = _build(layers, cfg, dev, dtype)
+    before = {u: store.buckets[u].flat_params.clone() for u in store.buckets}
+    out = ex.run(one_f_one_b(MB, [0, 1]), xs)
+    torch.cuda.synchronize()
+    assert len(out["losses"]) == MB and all(torch.isfinite(l) for l in out["losses"])
+    for u, b in store.buckets.items():
+        assert torch.isfinite(b.flat_grads).all() and float(b.flat_grads.abs().max()) > 0
+        st = b.shard_optimizer.state[b.shard_param]
+        assert st["step"] == 1
+        # parameters are views of the bucket the optimizer wrote, and the bucket moved
+        for (p, off, n, shape) in b.param_view_specs:
+            assert p.data_ptr() == b.flat_params.data_ptr() + off * b.flat_params.element_size() and p.grad is None
+        assert not torch.equal(before[u], b.flat_params)
+        # the update equals torch.optim.AdamW on a slice of the bucket, given the bucket's own gradient
+        n = min(b.flat_params.numel(), 1 << 20)
+        m0 = before[u][:n].float().cpu()
+        z = torch.zeros_like(m0)
+        want, _, _ = OB.adamw_step_torch(m0, b.flat_grads[:n].cpu(), z, z, 1, ADAMW["lr"], ADAMW["betas"], ADAMW["eps"],
+                                         ADAMW["weight_decay"])
+        assert (st["master"][:n].cpu() - want).abs().max().item() <= ADAMW_TOL
+    # every token contributed K rows to the experts of both layers: the expert gradients are dense
+    for ubid in (0, 1):
+        b = store.buckets[ubid]
+        spec = {name: s for s, name in zip(b.param_view_specs, names)}
+        p, off, n, shape = spec["w2"]
+        g = b.flat_grads[off:off + n].view(shape)
+        assert int((g.abs().amax(dim=(1, 2)) > 0).sum()) == cfg[4]
