@@ -262,6 +262,10 @@ PK_API int pk_adamw_fused(float* master, float* exp_avg, float* exp_avg_sq, floa
  * launch order, forgets them and returns how many launches were recorded. */
 PK_API int pk_timing_enable(int on);
 PK_API int64_t pk_timing_collect(int32_t* ids, float* ms, int64_t max_records);
+/* Restrict the bracketing to launches of one kernel id (as returned in `ids`); a negative id times
+ * every kernel again.  Two event records per launch cost the stream a few microseconds, which
+ * adds up over the ~20 launches of a step: a throughput measurement times only what it needs. */
+PK_API int pk_timing_select(int kernel_id);
 PK_API const char* pk_timing_kernel_name(int id);
 
 #ifdef __cplusplus

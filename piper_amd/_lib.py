@@ -58,6 +58,7 @@ SIGNATURES = {
                                 _c_f32, _c_i64, _c_f32, _c_int, _p]),
     "pk_timing_enable": (_c_int, [_c_int]),
     "pk_timing_collect": (_c_i64, [_p, _p, _c_i64]),
+    "pk_timing_select": (_c_int, [_c_int]),
     "pk_timing_kernel_name": (C.c_char_p, [_c_int]),
 }
 
@@ -101,6 +102,23 @@ def call(name: str, *args):
 def timing_enable(on: bool) -> None:
     """Switch per-kernel HIP-event timing inside the library on or off."""
     load().pk_timing_enable(int(bool(on)))
+
+
+def timing_select(name: str | None) -> None:
+    """Time only the kernel with this name (as timing_collect reports it); None times all again."""
+    lib = load()
+    kid = -1
+    if name is not None:
+        i = 0
+        while True:
+            n = lib.pk_timing_kernel_name(i).decode()
+            if n == "unknown":
+                raise ValueError(f"no kernel named {name!r}")
+            if n == name:
+                kid = i
+                break
+            i += 1
+    lib.pk_timing_select(kid)
 
 
 def timing_collect(max_records: int = 1 << 16) -> list[tuple[str, float]]:

@@ -11,6 +11,7 @@ namespace {
 struct Rec { int id; hipEvent_t start, stop; };
 std::mutex g_mu;
 bool g_on = false;
+int g_only = -1;   // >= 0: only launches of this kernel id are bracketed
 std::vector<Rec> g_recs;
 std::vector<hipEvent_t> g_pool;
 
@@ -31,7 +32,7 @@ const char* const kNames[K_COUNT] = {
 
 Scope::Scope(int id, hipStream_t s) : stream_(s), slot_(-1) {
   std::lock_guard<std::mutex> lk(g_mu);
-  if (!g_on) return;
+  if (!g_on || (g_only >= 0 && id != g_only)) return;
   Rec r{id, get_event(), get_event()};
   if (!r.start || !r.stop) return;
   if (hipEventRecord(r.start, s) != hipSuccess) return;
@@ -68,6 +69,12 @@ int64_t pk_timing_collect(int32_t* ids, float* ms, int64_t max_records) {
   }
   pk_timing::g_recs.clear();
   return n;
+}
+
+int pk_timing_select(int kernel_id) {
+  std::lock_guard<std::mutex> lk(pk_timing::g_mu);
+  pk_timing::g_only = (kernel_id >= 0 && kernel_id < pk_timing::K_COUNT) ? kernel_id : -1;
+  return PK_OK;
 }
 
 const char* pk_timing_kernel_name(int id) {
