@@ -59,9 +59,10 @@ def kernel_bytes(cfg) -> dict:
     return {
         "swiglu_gate_up": 2 * w + 2.0 * T * H + 3 * 2.0 * A * I,        # w1,w3 + x (each token once) -> g,u,h
         "swiglu_down": w + 2.0 * A * I + 2.0 * A * H,                   # w2 + h -> y
-        "swiglu_dgrad_dh": w + 2.0 * A * H + 2 * 2.0 * A * I + 2 * 2.0 * A * I,   # w2 + d_y + g,u -> d_g,d_u
+        # w2 + d_out (each token once) + g,u -> d_g,d_u,score*h (+ the score-gradient partials)
+        "swiglu_dgrad_dh": w + 2.0 * T * H + 2 * 2.0 * A * I + 3 * 2.0 * A * I + 4.0 * A * (I / 64),
         "swiglu_dgrad_dx": 2 * w + 2 * 2.0 * A * I + 2.0 * A * H,       # w1,w3 + d_g,d_u -> d_x rows
-        "swiglu_wgrad": 2.0 * A * H + 3 * 2.0 * A * I + 2.0 * T * H + 3 * w,      # d_y,h,d_g,d_u,x -> d_w1..3
+        "swiglu_wgrad": 2 * 2.0 * T * H + 3 * 2.0 * A * I + 3 * w,      # d_out,x (each token once), score*h,d_g,d_u -> d_w1..3
     }
 
 

@@ -195,6 +195,26 @@ PK_API int pk_grouped_swiglu_dgrad_dx(const void* d_g, const void* d_u, const vo
                                const int32_t* starts, void* d_x_sorted, int64_t A, int64_t H,
                                int64_t I, int64_t E, int dtype, pk_stream_t stream);
 
+/* Input gradient of the experts with the weighted combine folded in: what pk_combine_bwd followed
+ * by pk_grouped_swiglu_dgrad_dh computes (the backward of qwen3.py:268-289 up to the SwiGLU
+ * pre-activations), without materialising d_y = score * d_out[token] per routed row.
+ *   sorted row r belongs to flat slot m = row_map[r] (token m / row_map_div), score scores[m]
+ *   a[r]        = d_out[m / row_map_div] . w2[e]^T                     (fp32, never stored)
+ *   d_scores[m] = < a[r], silu(g[r]) * u[r] >                          ([T*K] f32, every slot written)
+ *   d_g, d_u    = SwiGLU backward of (scores[m] * a[r])                ([A,I], dtype)
+ *   hs[r]       = scores[m] * silu(g[r]) * u[r]                        ([A,I], dtype)
+ * hs replaces h and d_out replaces d_y in the weight gradient (pk_grouped_swiglu_wgrad_scaled):
+ * d_w2[e] = sum_r d_out[token_r]^T . hs[r].  The matrix-core path needs a workspace of
+ * pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes (partial score gradients per 64 columns,
+ * summed in a fixed order). */
+PK_API int64_t pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes(int64_t A, int64_t I);
+PK_API int pk_grouped_swiglu_dgrad_dh_scaled(const void* d_out, const int32_t* row_map, int64_t row_map_div,
+                                      const float* scores, const void* w2, const void* g,
+                                      const void* u, const int32_t* starts, void* d_g, void* d_u,
+                                      void* hs, float* d_scores, void* workspace,
+                                      int64_t workspace_bytes, int64_t A, int64_t H, int64_t I,
+                                      int64_t E, int dtype, pk_stream_t stream);
+
 /* Weight gradient (Piper's BWD_W task, src/executors.py:413-476).
  *   d_w2[e] (+)= d_y[rows_e]^T . h[rows_e]          [H,I]
  *   d_w1[e] (+)= d_g[rows_e]^T . x[rows_e]          [I,H]
@@ -211,6 +231,15 @@ PK_API int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d
                             void* d_w2, void* d_w3,
                             int accumulate, int64_t A, int64_t H, int64_t I, int64_t E,
                             int dtype, pk_stream_t stream);
+
+/* The same weight gradients from the outputs of pk_grouped_swiglu_dgrad_dh_scaled: d_out [T,H]
+ * is addressed through row_map / row_map_div like x, hs [A,I] takes the place of h. */
+PK_API int pk_grouped_swiglu_wgrad_scaled(const void* d_out, const void* hs, const void* d_g, const void* d_u,
+                                   const void* x, const int32_t* row_map, int64_t row_map_div,
+                                   const int32_t* starts, const int32_t* expert_order, void* d_w1,
+                                   void* d_w2, void* d_w3,
+                                   int accumulate, int64_t A, int64_t H, int64_t I, int64_t E,
+                                   int dtype, pk_stream_t stream);
 
 /* ------------------------------------------------------------- ZeRO bucket path */
 

@@ -50,6 +50,11 @@ SIGNATURES = {
     "pk_grouped_swiglu_dgrad_dx": (_c_int, [_p, _p, _p, _p, _p, _p, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
     "pk_grouped_swiglu_wgrad": (_c_int, [_p, _p, _p, _p, _p, _p, _c_i64, _p, _p, _p, _p, _p, _c_int,
                                          _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
+    "pk_grouped_swiglu_wgrad_scaled": (_c_int, [_p, _p, _p, _p, _p, _p, _c_i64, _p, _p, _p, _p, _p, _c_int,
+                                                _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
+    "pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes": (_c_i64, [_c_i64, _c_i64]),
+    "pk_grouped_swiglu_dgrad_dh_scaled": (_c_int, [_p, _p, _c_i64, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _c_i64,
+                                                   _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
     "pk_bucket_plan": (_c_i64, [_p, _c_i64, _c_i64, _c_i64, _p]),
     "pk_bucket_pack": (_c_int, [_p, _p, _p, _c_i64, _c_int, _p, _c_int, _c_int, _p]),
     "pk_bucket_unpack": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_int, _p]),

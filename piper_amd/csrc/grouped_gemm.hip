@@ -21,7 +21,10 @@ namespace mf {
 constexpr int NXCD = 8;
 
 
-enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_SWIGLU_BWD = 2 };
+// EPI_SWIGLU_BWD_SCALED: the A rows are rows of d_out gathered through the row map, the
+// accumulator is the unscaled d_h; the epilogue multiplies by the row's combine score, also
+// emits score * h and the per-row partial dot products <unscaled d_h, h> (the score gradient).
+enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_SWIGLU_BWD = 2, EPI_SWIGLU_BWD_SCALED = 3 };
 
 typedef short shortx4_t __attribute__((ext_vector_type(4)));
 // Read-only tables (row offsets, row maps) addressed wave-uniformly: going through the constant
@@ -397,8 +400,11 @@ struct RaggedMParams {
   const bf16_t* Uin;
   bf16_t* O0;            // PLAIN: C;  SWIGLU: g;  SWIGLU_BWD: d_g
   bf16_t* O1;            //            SWIGLU: u;  SWIGLU_BWD: d_u
-  bf16_t* O2;            //            SWIGLU: h
+  bf16_t* O2;            //            SWIGLU: h;  SWIGLU_BWD_SCALED: score * h
   int64_t ldc;
+  const float* scores;   // SWIGLU_BWD_SCALED: score of sorted row r is scores[row_map[r]]
+  float* ds_partial;     // SWIGLU_BWD_SCALED: [ldc / 64][total_rows] partial <unscaled d_h, h>
+  int64_t total_rows;
   SchedSlot* sched;      // this launch's counters
 #ifdef PK_GEMM_DEBUG
   int32_t debug;         // 1: skip MFMAs, 2: skip loads, 4: skip stores
@@ -512,6 +518,9 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   constexpr int LA = A_BYTES / (NTHREADS * 16), LB = (STAGE - A_BYTES) / (NTHREADS * 16), L = LA + LB;
   static_assert(LA >= 1 && LB >= 1 && TM >= 1 && TN >= 1, "tile too small for the wave grid");
   static_assert(EPI != EPI_SWIGLU || (WTN % 64 == 0), "gate/up pairs must stay inside a wave");
+  static_assert(EPI != EPI_SWIGLU_BWD_SCALED || WTN == 64, "one score-gradient partial per 64 columns");
+  constexpr bool BWD = EPI == EPI_SWIGLU_BWD || EPI == EPI_SWIGLU_BWD_SCALED;
+  constexpr bool SCALED = EPI == EPI_SWIGLU_BWD_SCALED;
   constexpr int OUT_COLS = (EPI == EPI_SWIGLU) ? WTN / 2 : WTN;   // columns a wave writes per output tensor
   constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;       // output columns per tile
   using St = Stage32<OUT_COLS>;
@@ -694,7 +703,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
           if (s < nkt && dbg_loads) issue_tile(nxt_u, s, cur + s >= NS ? cur + s - NS : cur + s);
       }
     };
-    if (EPI != EPI_SWIGLU_BWD) prefetch_next();
+    if (!BWD) prefetch_next();
 
     // ---- epilogue, 32 rows of the wave tile at a time through the wave's staging buffer
     const int lrow = lane & 31, lq = 4 * (lane >> 5);
@@ -746,18 +755,21 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
           st_after += St::template flush<false>(sbuf, p.O0 + goff, p.ldc, crows);
           wave_lds_fence();
         }
-      } else {   // EPI_SWIGLU_BWD: acc = d_h; d_g = d_h * u * silu'(g), d_u = d_h * silu(g)
-        u32x2_t dg[TN][4], du[TN][4];
+      } else {   // EPI_SWIGLU_BWD[_SCALED]: acc = d_h; d_g = d_h * u * silu'(g), d_u = d_h * silu(g)
+        u32x2_t dg[TN][4], du[TN][4], hs[SCALED ? TN : 1][4];
+        float ds = 0.f;
         if (crows > 0) {
           const int rr = lrow < crows ? lrow : crows - 1;
+          float sc = 1.f;
+          if (SCALED) sc = p.scores[p.row_map[cur_u.row0 + wm * WTM + 32 * i + rr]];
 #pragma unroll
           for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               const int64_t off = goff + (int64_t)rr * p.ldc + 32 * j + 8 * q + lq;
-              float dh[4], g[4], u[4], og[4], ou[4];
+              float dh[4], g[4], u[4], og[4], ou[4], oh[4];
               // d_h is rounded to bf16 first, like the output of the reference's batched matmul
-              unpack4(pack4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]), dh);
+              unpack4(pack4(sc * acc[i][j][4 * q], sc * acc[i][j][4 * q + 1], sc * acc[i][j][4 * q + 2], sc * acc[i][j][4 * q + 3]), dh);
               unpack4(*reinterpret_cast<const u32x2_t*>(p.Gin + off), g);
               unpack4(*reinterpret_cast<const u32x2_t*>(p.Uin + off), u);
 #pragma unroll
@@ -765,23 +777,37 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
                 const float sg = 1.f / (1.f + __expf(-g[t]));
                 og[t] = dh[t] * u[t] * (sg * (1.f + g[t] * (1.f - sg)));
                 ou[t] = dh[t] * (g[t] * sg);
+                if (SCALED) {
+                  const float hv = (g[t] * sg) * u[t];
+                  ds += acc[i][j][4 * q + t] * hv;
+                  oh[t] = sc * hv;
+                }
               }
               dg[j][q] = pack4(og[0], og[1], og[2], og[3]);
               du[j][q] = pack4(ou[0], ou[1], ou[2], ou[3]);
+              if (SCALED) hs[j][q] = pack4(oh[0], oh[1], oh[2], oh[3]);
             }
         }
         // the loads above must have returned first: a load behind the prefetch waits for all of it
         __builtin_amdgcn_sched_barrier(0);
         if (i == TM - 1) prefetch_next();
         if (crows > 0 && do_store) {
+          if (SCALED) {
+            // lanes l and l+32 hold the two column halves of row l % 32
+            ds += __shfl_xor(ds, 32);
+            if (lane < 32 && lrow < crows)
+              p.ds_partial[(int64_t)((cur_u.nt * BN + wn * WTN) >> 6) * p.total_rows + cur_u.row0 + wm * WTM + 32 * i + lrow] = ds;
+            st_after += 1;
+          }
 #pragma unroll
-          for (int which = 0; which < 2; ++which) {
+          for (int which = 0; which < (SCALED ? 3 : 2); ++which) {
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
-              for (int q = 0; q < 4; ++q) St::put(sbuf, lrow, 32 * j + 8 * q + lq, which == 0 ? dg[j][q] : du[j][q]);
+              for (int q = 0; q < 4; ++q)
+                St::put(sbuf, lrow, 32 * j + 8 * q + lq, which == 0 ? dg[j][q] : which == 1 ? du[j][q] : hs[SCALED ? j : 0][q]);
             wave_lds_fence();
-            st_after += St::template flush<false>(sbuf, (which == 0 ? p.O0 : p.O1) + goff, p.ldc, crows);
+            st_after += St::template flush<false>(sbuf, (which == 0 ? p.O0 : which == 1 ? p.O1 : p.O2) + goff, p.ldc, crows);
             wave_lds_fence();
           }
         }
@@ -1026,6 +1052,46 @@ __global__ void swiglu_bwd_kernel(const T* dh, const T* __restrict__ g,
   }
 }
 
+// Sum the per-64-column partials of the score gradient and store them at the flat (token, k)
+// slot of each sorted row.
+__global__ void dscore_reduce_kernel(const float* __restrict__ part, int P, int64_t A,
+                                     const int32_t* __restrict__ row_map, float* __restrict__ d_scores) {
+  const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= A) return;
+  float s = 0.f;
+  for (int q = 0; q < P; ++q) s += part[(int64_t)q * A + r];
+  d_scores[row_map[r]] = s;
+}
+
+// Generic second half of the scaled SwiGLU backward: one wave per sorted row.  dh holds the
+// unscaled d_h = d_out[token] . w2 and may alias du.
+template <typename T>
+__global__ void swiglu_bwd_scaled_rows_kernel(const T* dh, const T* __restrict__ g, const T* __restrict__ u,
+                                              const int32_t* __restrict__ row_map, const float* __restrict__ scores,
+                                              T* __restrict__ dg, T* du, T* __restrict__ hs,
+                                              float* __restrict__ d_scores, int64_t A, int64_t I) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (r >= A) return;
+  const int slot = row_map[r];
+  const float sc = scores[slot];
+  float ds = 0.f;
+  for (int64_t i = lane; i < I; i += 64) {
+    const int64_t o = r * I + i;
+    const float a = pk_to_float<T>(dh[o]), gv = pk_to_float<T>(g[o]), uv = pk_to_float<T>(u[o]);
+    const float sg = 1.f / (1.f + expf(-gv));
+    const float hv = (gv * sg) * uv;
+    ds += a * hv;
+    const float d = pk_to_float<T>(pk_from_float<T>(sc * a));
+    dg[o] = pk_from_float<T>(d * uv * (sg * (1.f + gv * (1.f - sg))));
+    du[o] = pk_from_float<T>(d * (gv * sg));
+    hs[o] = pk_from_float<T>(sc * hv);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) ds += __shfl_xor(ds, off);
+  if (lane == 0) d_scores[slot] = ds;
+}
+
 // Generic (any shape) ragged GEMMs on the FMA kernel.  T = element type of every operand.
 template <typename T>
 int simt_ragged_m(const void* A, int64_t lda, const int32_t* row_map, int64_t map_div,
@@ -1127,11 +1193,11 @@ int fwd_simt(const void* x, const int32_t* row_map, int64_t div, const void* w1,
 }
 
 template <typename T>
-int wgrad_simt(const void* dy, const void* h, const void* dg, const void* du, const void* x,
+int wgrad_simt(const void* dy, const int32_t* dy_map, const void* h, const void* dg, const void* du, const void* x,
                const int32_t* row_map, int64_t div, const int32_t* starts, void* dw1, void* dw2,
                void* dw3, int acc, int64_t H, int64_t I, int64_t E, hipStream_t s) {
   int rc = PK_OK;
-  if (dw2) rc = simt_ragged_k<T>(dy, H, nullptr, h, I, nullptr, 1, dw2, starts, H, I, E, acc, s);
+  if (dw2) rc = simt_ragged_k<T>(dy, H, dy_map, h, I, nullptr, dy_map ? div : 1, dw2, starts, H, I, E, acc, s);
   if (rc) return rc;
   if (dw1) rc = simt_ragged_k<T>(dg, I, nullptr, x, H, row_map, div, dw1, starts, I, H, E, acc, s);
   if (rc) return rc;
@@ -1212,6 +1278,57 @@ int pk_grouped_swiglu_dgrad_dh(const void* d_y, const void* w2, const void* g, c
   return launch_rm<false, mf::EPI_SWIGLU_BWD>(p, A, I, pk_timing::K_SWIGLU_DGRAD_DH, s);
 }
 
+int64_t pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes(int64_t A, int64_t I) {
+  if (A < 0 || I <= 0) return PK_ERR_ARG;
+  return pk_ceil_div(I, 64) * A * (int64_t)sizeof(float);
+}
+
+int pk_grouped_swiglu_dgrad_dh_scaled(const void* d_out, const int32_t* row_map, int64_t row_map_div,
+                                      const float* scores, const void* w2, const void* g,
+                                      const void* u, const int32_t* starts, void* d_g, void* d_u,
+                                      void* hs, float* d_scores, void* workspace,
+                                      int64_t workspace_bytes, int64_t A, int64_t H, int64_t I,
+                                      int64_t E, int dtype, pk_stream_t stream) {
+  int rc = check_common(A, H, I, E, dtype);
+  if (rc) return rc;
+  if (A == 0) return PK_OK;
+  if (!d_out || !row_map || row_map_div <= 0 || !scores || !w2 || !g || !u || !starts || !d_g || !d_u || !hs || !d_scores)
+    return PK_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const bool simt = dtype == PK_F32 || !mfma_shape_ok(H, I) || !all_aligned16({d_out, w2, g, u, d_g, d_u, hs});
+  if (simt) {
+    // unscaled d_h = d_out[token] . w2[e], staged in d_u's buffer; then one wave per row
+    if (dtype == PK_F32) rc = simt_ragged_m<float>(d_out, H, row_map, row_map_div, w2, I, 1, H * I, d_u, I, starts, A, I, H, E, 0, s);
+    else rc = simt_ragged_m<bf16_t>(d_out, H, row_map, row_map_div, w2, I, 1, H * I, d_u, I, starts, A, I, H, E, 0, s);
+    if (rc) return rc;
+    const dim3 grid((unsigned)pk_ceil_div(A, 4)), block(256);
+    if (dtype == PK_F32)
+      PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_ELEMENTWISE, s, (swiglu_bwd_scaled_rows_kernel<float>), grid, block, 0, s,
+                        (const float*)d_u, (const float*)g, (const float*)u, row_map, scores, (float*)d_g, (float*)d_u, (float*)hs, d_scores, A, I);
+    else
+      PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_ELEMENTWISE, s, (swiglu_bwd_scaled_rows_kernel<bf16_t>), grid, block, 0, s,
+                        (const bf16_t*)d_u, (const bf16_t*)g, (const bf16_t*)u, row_map, scores, (bf16_t*)d_g, (bf16_t*)d_u, (bf16_t*)hs, d_scores, A, I);
+    PK_RETURN_IF_LAUNCH_FAILED();
+    return PK_OK;
+  }
+  const int64_t need = pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes(A, I);
+  if (!workspace || workspace_bytes < need) return PK_ERR_WORKSPACE;
+  mf::RaggedMParams p = {};
+  p.A0 = (const bf16_t*)d_out; p.lda = H;
+  p.row_map = row_map; p.map_div = (int32_t)row_map_div;
+  p.B0 = (const bf16_t*)w2; p.ldb = I; p.strideB = H * I;
+  p.starts = starts; p.E = (int32_t)E; p.Kseg = (int32_t)H; p.nseg = 1;
+  p.Gin = (const bf16_t*)g; p.Uin = (const bf16_t*)u;
+  p.O0 = (bf16_t*)d_g; p.O1 = (bf16_t*)d_u; p.O2 = (bf16_t*)hs; p.ldc = I;
+  p.scores = scores; p.ds_partial = (float*)workspace; p.total_rows = A;
+  rc = launch_rm<false, mf::EPI_SWIGLU_BWD_SCALED>(p, A, I, pk_timing::K_SWIGLU_DGRAD_DH, s);
+  if (rc) return rc;
+  PK_LAUNCH_NOCHECK(pk_timing::K_COMBINE_BWD, s, dscore_reduce_kernel, dim3((unsigned)pk_ceil_div(A, 256)), dim3(256), 0, s,
+                    (const float*)workspace, (int)(I / 64), A, row_map, d_scores);
+  PK_RETURN_IF_LAUNCH_FAILED();
+  return PK_OK;
+}
+
 int pk_grouped_swiglu_dgrad_dx(const void* d_g, const void* d_u, const void* w1, const void* w3,
                                const int32_t* starts, void* d_x_sorted, int64_t A, int64_t H,
                                int64_t I, int64_t E, int dtype, pk_stream_t stream) {
@@ -1250,12 +1367,13 @@ int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, con
   return pk_grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts, d_x_sorted, A, H, I, E, dtype, stream);
 }
 
-int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, const void* d_u,
-                            const void* x_rows, const int32_t* row_map, int64_t row_map_div,
-                            const int32_t* starts, const int32_t* expert_order, void* d_w1,
-                            void* d_w2, void* d_w3,
-                            int accumulate, int64_t A, int64_t H, int64_t I, int64_t E,
-                            int dtype, pk_stream_t stream) {
+// d_y rows are addressed directly (dy_gathered == 0) or through the row map like x
+static int wgrad_impl(const void* d_y, int dy_gathered, const void* h, const void* d_g, const void* d_u,
+                      const void* x_rows, const int32_t* row_map, int64_t row_map_div,
+                      const int32_t* starts, const int32_t* expert_order, void* d_w1,
+                      void* d_w2, void* d_w3,
+                      int accumulate, int64_t A, int64_t H, int64_t I, int64_t E,
+                      int dtype, pk_stream_t stream) {
   int rc = check_common(A, H, I, E, dtype);
   if (rc) return rc;
   if (!starts) return PK_ERR_ARG;
@@ -1263,18 +1381,20 @@ int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, con
   if (d_w1 && A > 0 && (!d_g || !x_rows)) return PK_ERR_ARG;
   if (d_w3 && A > 0 && (!d_u || !x_rows)) return PK_ERR_ARG;
   if (row_map && row_map_div <= 0) return PK_ERR_ARG;
+  if (dy_gathered && !row_map) return PK_ERR_ARG;
   if (!row_map) row_map_div = 1;
+  const int32_t* dy_map = dy_gathered ? row_map : nullptr;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PK_F32)
-    return wgrad_simt<float>(d_y, h, d_g, d_u, x_rows, row_map, row_map_div, starts, d_w1, d_w2, d_w3, accumulate, H, I, E, s);
+    return wgrad_simt<float>(d_y, dy_map, h, d_g, d_u, x_rows, row_map, row_map_div, starts, d_w1, d_w2, d_w3, accumulate, H, I, E, s);
   if (!mfma_shape_ok(H, I) || !all_aligned16({d_y, h, d_g, d_u, x_rows, d_w1, d_w2, d_w3}))
-    return wgrad_simt<bf16_t>(d_y, h, d_g, d_u, x_rows, row_map, row_map_div, starts, d_w1, d_w2, d_w3, accumulate, H, I, E, s);
+    return wgrad_simt<bf16_t>(d_y, dy_map, h, d_g, d_u, x_rows, row_map, row_map_div, starts, d_w1, d_w2, d_w3, accumulate, H, I, E, s);
 
   mf::WgradParams p = {};
   int n = 0;
   if (d_w2) {
     mf::WgradProblem& q = p.prob[n++];
-    q.A = (const bf16_t*)d_y; q.lda = H; q.a_map = nullptr;
+    q.A = (const bf16_t*)d_y; q.lda = H; q.a_map = dy_map;
     q.B = (const bf16_t*)h; q.ldb = I; q.b_map = nullptr;
     q.C = (bf16_t*)d_w2; q.M = (int32_t)H; q.N = (int32_t)I;
   }
@@ -1307,6 +1427,26 @@ int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, con
     PK_LAUNCH_NOCHECK(pk_timing::K_SWIGLU_WGRAD, s, (mf::wgrad_kernel<PK_WG_SMALL>), dim3((unsigned)blocks, n), dim3(PK_WG_SMALL_THREADS), 0, s, p);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
+}
+
+int pk_grouped_swiglu_wgrad(const void* d_y, const void* h, const void* d_g, const void* d_u,
+                            const void* x_rows, const int32_t* row_map, int64_t row_map_div,
+                            const int32_t* starts, const int32_t* expert_order, void* d_w1,
+                            void* d_w2, void* d_w3,
+                            int accumulate, int64_t A, int64_t H, int64_t I, int64_t E,
+                            int dtype, pk_stream_t stream) {
+  return wgrad_impl(d_y, 0, h, d_g, d_u, x_rows, row_map, row_map_div, starts, expert_order, d_w1, d_w2, d_w3,
+                    accumulate, A, H, I, E, dtype, stream);
+}
+
+int pk_grouped_swiglu_wgrad_scaled(const void* d_out, const void* hs, const void* d_g, const void* d_u,
+                                   const void* x, const int32_t* row_map, int64_t row_map_div,
+                                   const int32_t* starts, const int32_t* expert_order, void* d_w1,
+                                   void* d_w2, void* d_w3,
+                                   int accumulate, int64_t A, int64_t H, int64_t I, int64_t E,
+                                   int dtype, pk_stream_t stream) {
+  return wgrad_impl(d_out, 1, hs, d_g, d_u, x, row_map, row_map_div, starts, expert_order, d_w1, d_w2, d_w3,
+                    accumulate, A, H, I, E, dtype, stream);
 }
 
 }  // extern "C"

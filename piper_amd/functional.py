@@ -104,17 +104,18 @@ class _BmmExpertsFn(torch.autograd.Function):
         return d_w1, d_w2, d_w3, d_x, None
 
 
-def _queue_expert_wgrad(params, d_y, h, d_g, d_u, x, starts, perm, top_k, order) -> None:
+def _queue_expert_wgrad(params, d_y, h, d_g, d_u, x, starts, perm, top_k, order, scaled=False) -> None:
     p1, p2, p3 = params
 
     def run():
         bufs = [_grad_target(p) for p in (p1, p2, p3)]
         if all(acc for _, acc in bufs):     # accumulate in the kernel's epilogue
             ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, p1.shape[0], row_map=perm, row_map_div=top_k,
-                                     expert_order=order, d_w1=bufs[0][0], d_w2=bufs[1][0], d_w3=bufs[2][0], accumulate=True)
+                                     expert_order=order, d_w1=bufs[0][0], d_w2=bufs[1][0], d_w3=bufs[2][0], accumulate=True,
+                                     scaled=scaled)
             return
         g1, g2, g3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, p1.shape[0], row_map=perm,
-                                              row_map_div=top_k, expert_order=order)
+                                              row_map_div=top_k, expert_order=order, scaled=scaled)
         for p, g in ((p1, g1), (p2, g2), (p3, g3)):
             if p.grad is None:
                 p.grad = g
@@ -276,19 +277,24 @@ class _ExpertRegionFn(torch.autograd.Function):
         _counts, starts, perm, inv_perm, order = ops.sort_by_expert(top_idx, E, with_order=True)
         y, g, u, h = ops.grouped_swiglu_fwd(x, w1, w2, w3, starts, row_map=perm, row_map_div=top_k)
         out = ops.combine_fwd(y, inv_perm, top_scores, residual)
-        ctx.save_for_backward(x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, h, y, order)
+        # the backward recomputes h from (g, u) and takes the score gradient from the d_h GEMM, so
+        # neither h nor y outlives the forward
+        ctx.save_for_backward(x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, order)
         ctx.cfg = (top_k, route_norm, route_scale, gate_bias is not None)
         ctx.params = (w_gate, gate_bias, w1, w2, w3)
         return out
 
     @staticmethod
     def backward(ctx, d_out):
-        (x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, h, y, order) = ctx.saved_tensors
+        (x, w_gate, w1, w2, w3, logits, top_scores, top_idx, starts, perm, inv_perm, g, u, order) = ctx.saved_tensors
         top_k, route_norm, route_scale, has_bias = ctx.cfg
         E = w1.shape[0]
         need = ctx.needs_input_grad
-        d_y, d_scores = ops.combine_bwd(d_out, y, perm, top_scores)
-        d_g, d_u = ops.grouped_swiglu_dgrad_dh(d_y, w2, g, u, starts)
+        # combine backward folded into the d_h GEMM: d_out rows are gathered per routed row, the
+        # score is applied in the epilogue; d_y below is d_out itself and h is score * h
+        d_out = d_out.contiguous()
+        d_g, d_u, h, d_scores = ops.grouped_swiglu_dgrad_dh_scaled(d_out, perm, top_scores, w2, g, u, starts)
+        d_y = d_out
         # The weight gradient (Piper's BWD_W) depends only on d_y, h, d_g, d_u and x; it runs on a
         # second stream next to the input gradient (BWD_I) so the two kernels fill each other's tails.
         d_w1 = d_w2 = d_w3 = None
@@ -298,7 +304,7 @@ class _ExpertRegionFn(torch.autograd.Function):
             # backward-input pass: the weight gradients of the experts and of the router gate are
             # queued with the tensors they need and computed by the weight pass
             p_gate, p_bias = ctx.params[0], ctx.params[1]
-            _queue_expert_wgrad(ctx.params[2:], d_y, h, d_g, d_u, x, starts, perm, top_k, order)
+            _queue_expert_wgrad(ctx.params[2:], d_y, h, d_g, d_u, x, starts, perm, top_k, order, scaled=True)
             d_xs = ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
             d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
             d_x32 = ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=need[0], d_w_gate=None, d_gate_bias=None)
@@ -325,9 +331,9 @@ class _ExpertRegionFn(torch.autograd.Function):
             if side is not None:
                 side.wait_stream(cur)
                 with torch.cuda.stream(side):
-                    d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k, expert_order=order)
+                    d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k, expert_order=order, scaled=True)
             else:
-                d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k, expert_order=order)
+                d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k, expert_order=order, scaled=True)
         d_xs = ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
         d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
         d_wg = torch.empty_like(w_gate) if need[1] else None
@@ -336,7 +342,7 @@ class _ExpertRegionFn(torch.autograd.Function):
         d_x = ops.permute_bwd(d_xs, inv_perm, top_k, addend_f32=d_x32) if need[0] else None
         if side is not None:
             cur.wait_stream(side)
-            for t in (d_y, d_g, d_u):        # allocated on the current stream, read on the side stream
+            for t in (d_y, h, d_g, d_u):     # allocated on the current stream, read on the side stream
                 t.record_stream(side)
             for t in (d_w1, d_w2, d_w3):     # allocated on the side stream, consumed on the current one
                 t.record_stream(cur)

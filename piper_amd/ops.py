@@ -255,6 +255,27 @@ def grouped_swiglu_dgrad_dh(d_y, w2, g, u, starts):
     return d_g, d_u
 
 
+def grouped_swiglu_dgrad_dh_scaled(d_out, perm, top_scores, w2, g, u, starts):
+    """combine_bwd + grouped_swiglu_dgrad_dh in one GEMM launch, without the per-row d_y:
+    returns (d_g, d_u, hs = score * h [A,I], d_scores [T,K] f32).  Sorted row r is flat slot perm[r] of
+    top_scores [T,K] and token perm[r] // K of d_out [T,H]."""
+    require_gpu(d_out)
+    E, H, I = w2.shape
+    A = perm.numel()
+    T, K = top_scores.shape
+    dev = d_out.device
+    d_g = torch.empty_like(g)
+    d_u = torch.empty_like(u)
+    hs = torch.empty_like(g)
+    d_scores = torch.empty((T, K), dtype=torch.float32, device=dev)
+    ws_bytes = int(_lib.load().pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes(A, I))
+    ws = torch.empty(max(ws_bytes, 4) // 4, dtype=torch.float32, device=dev)
+    call("pk_grouped_swiglu_dgrad_dh_scaled", ptr(d_out.contiguous()), ptr(perm), K, ptr(top_scores.contiguous()),
+         ptr(w2.contiguous()), ptr(g), ptr(u), ptr(starts), ptr(d_g), ptr(d_u), ptr(hs), ptr(d_scores), ptr(ws), ws_bytes,
+         A, H, I, E, dtype_code(g.dtype), current_stream(dev))
+    return d_g, d_u, hs, d_scores
+
+
 def grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts):
     """Second half of the input gradient: d_x_sorted [A,H] = d_g . w1 + d_u . w3."""
     require_gpu(d_g)
@@ -267,19 +288,22 @@ def grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts):
 
 
 def grouped_swiglu_wgrad(d_y, h, d_g, d_u, x_rows, starts, E, *, row_map=None, row_map_div=1,
-                         d_w1=None, d_w2=None, d_w3=None, accumulate=False, expert_order=None):
+                         d_w1=None, d_w2=None, d_w3=None, accumulate=False, expert_order=None, scaled=False):
     """Weight gradients.  Without d_w* buffers, fresh tensors are returned; with buffers and
-    accumulate=True the kernel adds into them (gradient accumulation over microbatches)."""
+    accumulate=True the kernel adds into them (gradient accumulation over microbatches).
+    scaled=True: d_y is d_out [T,H], addressed through the row map like x_rows, and h is score * h
+    (the outputs of grouped_swiglu_dgrad_dh_scaled)."""
     require_gpu(d_y)
-    A, H = d_y.shape
-    I = h.shape[1]
+    A, I = h.shape
+    H = d_y.shape[1]
+    _check(not scaled or row_map is not None, "scaled weight gradient needs the row map")
     dt, dev = d_y.dtype, d_y.device
     if d_w1 is None:
         d_w1 = torch.empty((E, I, H), dtype=dt, device=dev)
         d_w2 = torch.empty((E, H, I), dtype=dt, device=dev)
         d_w3 = torch.empty((E, I, H), dtype=dt, device=dev)
         accumulate = False
-    call("pk_grouped_swiglu_wgrad", ptr(d_y.contiguous()), ptr(h), ptr(d_g), ptr(d_u), ptr(x_rows.contiguous()),
+    call("pk_grouped_swiglu_wgrad_scaled" if scaled else "pk_grouped_swiglu_wgrad", ptr(d_y.contiguous()), ptr(h), ptr(d_g), ptr(d_u), ptr(x_rows.contiguous()),
          ptr(row_map), row_map_div, ptr(starts), ptr(expert_order), ptr(d_w1), ptr(d_w2), ptr(d_w3), int(bool(accumulate)),
          A, H, I, E, dtype_code(dt), current_stream(dev))
     return d_w1, d_w2, d_w3

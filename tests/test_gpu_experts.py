@@ -71,6 +71,57 @@ def test_grouped_swiglu_fwd_dgrad_wgrad(dev, dtype, counts, H, I):
     assert rel_err(dw2, 2 * dw2_ref) <= tol and rel_err(dw1, 2 * dw1_ref) <= tol
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("counts,H,I", CASES + [([10, 0, 70, 3, 1], 192, 64)])
+def test_scaled_backward_matches_combine_bwd_then_dgrad(dev, dtype, counts, H, I):
+    """The backward with the weighted combine folded into the d_h GEMM (d_out rows gathered, score
+    applied in the epilogue, score gradient from the same accumulator) against the unfused chain
+    combine_bwd -> dgrad_dh -> wgrad, and against fp32 autograd through the oracle."""
+    print(f"[case] scaled backward {dtype} counts={counts[:8]} H={H} I={I}", flush=True)
+    K = 2
+    A = int(sum(counts))
+    assert A % K == 0
+    T, E = A // K, len(counts)
+    gen = torch.Generator().manual_seed(11)
+    _, w1, w2, w3, _, cnt = _make(5, counts, H, I, dtype)
+    perm = torch.randperm(A, generator=gen).to(torch.int32)          # sorted row -> flat (token, k) slot
+    tok = perm.long() // K
+    x_tok = torch.randn(T, H, generator=gen).to(dtype)
+    x_sorted = x_tok[tok]
+    scores = torch.rand(T, K, generator=gen) + 0.1
+    d_out = torch.randn(T, H, generator=gen).to(dtype)
+    tol = BF16_TOL if dtype == torch.bfloat16 else F32_TOL
+
+    XT, XS, W1, W2, W3, PERM, SC, DO = (t.to(dev) for t in (x_tok, x_sorted, w1, w2, w3, perm, scores, d_out))
+    starts = ops.counts_to_starts(cnt.to(dev))
+    y, g, u, h = ops.grouped_swiglu_fwd(XT, W1, W2, W3, starts, row_map=PERM, row_map_div=K)
+
+    # fp32 reference: out[t] = sum_k s[t,k] * y[row(t,k)]
+    xr, w1r, w2r, w3r = (t.float().requires_grad_(True) for t in (x_sorted, w1, w2, w3))
+    sr = scores.clone().requires_grad_(True)
+    y_ref = O.grouped_swiglu(w1r, w2r, w3r, xr, cnt)
+    out_ref = torch.zeros(T, H).index_add(0, tok, y_ref * sr.reshape(-1)[perm.long()].unsqueeze(1))
+    dx_ref, dw1_ref, dw2_ref, dw3_ref, ds_ref = torch.autograd.grad(out_ref, (xr, w1r, w2r, w3r, sr), d_out.float())
+
+    d_g, d_u, hs, d_s = ops.grouped_swiglu_dgrad_dh_scaled(DO, PERM, SC, W2, g, u, starts)
+    assert d_s.shape == (T, K) and rel_err(d_s, ds_ref) <= tol
+    d_xs = ops.grouped_swiglu_dgrad_dx(d_g, d_u, W1, W3, starts)
+    assert rel_err(d_xs, dx_ref) <= tol
+    dw1, dw2, dw3 = ops.grouped_swiglu_wgrad(DO, hs, d_g, d_u, XT, starts, E, row_map=PERM, row_map_div=K, scaled=True)
+    assert rel_err(dw1, dw1_ref) <= tol and rel_err(dw2, dw2_ref) <= tol and rel_err(dw3, dw3_ref) <= tol
+
+    # the unfused chain on the same inputs
+    d_y, d_s2 = ops.combine_bwd(DO, y, PERM, SC)
+    d_g2, d_u2 = ops.grouped_swiglu_dgrad_dh(d_y, W2, g, u, starts)
+    loose = 2 * tol          # both sides round at different places
+    assert rel_err(d_s, d_s2) <= loose and rel_err(d_g, d_g2) <= loose and rel_err(d_u, d_u2) <= loose
+    _, dw2_b, _ = ops.grouped_swiglu_wgrad(d_y, h, d_g2, d_u2, XS, starts, E)
+    assert rel_err(dw2, dw2_b) <= loose
+    for e, c in enumerate(counts):
+        if c == 0:
+            assert float(dw2[e].abs().max()) == 0.0
+
+
 def test_mfma_path_agrees_with_fma_path(dev):
     """bf16 shapes outside the MFMA tiling (H or I not a multiple of 128) run on the FMA kernel."""
     print("[case] bf16 fallback shapes", flush=True)
