@@ -463,18 +463,27 @@ struct Stage32 {
 // swapped (B first) so that a lane's accumulator holds 4 CONSECUTIVE columns of ONE row:
 //   acc[i][j][v] = C[row = 32*i + lane%32][col = 32*j + 8*(v/4) + 4*(lane/32) + v%4]
 template <int BK, int TM, int TN, bool A_KC, bool B_KC, int ACOLS, int BCOLS, int L, typename F>
-__device__ __forceinline__ void mma_ktile(const char* At, const char* Bt, int wrow0, int wcol0,
+__device__ __forceinline__ void mma_ktile(const char* At, const char* Bt, const char* At_next, const char* Bt_next,
+                                          bool has_next_tile, int wrow0, int wcol0, Frags<TM, TN>& f0,
                                           floatx16_t (&acc)[TM][TN], bool do_issue, F&& issue_one) {
   const int lane = threadIdx.x & 63;
   constexpr int KS = BK / 16, NM = KS * TM * TN;
   constexpr int EVERY = NM / L > 0 ? NM / L : 1;
   static_assert(L <= NM, "more loads than MFMAs in a k-tile");
   static_assert(TM + TN <= TM * TN, "one fragment read per MFMA slot");
+  static_assert(KS % 2 == 0, "the fragments handed to the next k-tile live in buffer 0");
+  // f0 holds the fragments of this tile's first k-step (read during the previous tile, or by
+  // the caller for a unit's first tile); on return it holds those of the next tile, whose
+  // operands the caller has made visible before this call
   Frags<TM, TN> f[2];
-  load_frags<BK, TM, TN, A_KC, B_KC, ACOLS, BCOLS>(f[0], At, Bt, wrow0, wcol0, 0, lane);
+  f[0] = f0;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     __builtin_amdgcn_sched_barrier(0);
+    const bool last = ks + 1 == KS;
+    const char* An = last ? At_next : At;
+    const char* Bn = last ? Bt_next : Bt;
+    const int ksn = last ? 0 : ks + 1;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -484,12 +493,12 @@ __device__ __forceinline__ void mma_ktile(const char* At, const char* Bt, int wr
         // k-step starts with row 0) and at most one load behind each MFMA
         __builtin_amdgcn_sched_barrier(0);
         const int m = i * TN + j;
-        if (ks + 1 < KS) {
+        if (!last || has_next_tile) {
           if (m < TN)
-            f[(ks + 1) & 1].b[m] = B_KC ? frag_kc<BK>(Bt, wcol0 + 32 * m, ks + 1, lane) : frag_mn<BCOLS>(Bt, wcol0 + 32 * m, ks + 1, lane);
+            f[(ks + 1) & 1].b[m] = B_KC ? frag_kc<BK>(Bn, wcol0 + 32 * m, ksn, lane) : frag_mn<BCOLS>(Bn, wcol0 + 32 * m, ksn, lane);
           else if (m < TN + TM)
-            f[(ks + 1) & 1].a[m - TN] = A_KC ? frag_kc<BK>(At, wrow0 + 32 * (m - TN), ks + 1, lane)
-                                             : frag_mn<ACOLS>(At, wrow0 + 32 * (m - TN), ks + 1, lane);
+            f[(ks + 1) & 1].a[m - TN] = A_KC ? frag_kc<BK>(An, wrow0 + 32 * (m - TN), ksn, lane)
+                                             : frag_mn<ACOLS>(An, wrow0 + 32 * (m - TN), ksn, lane);
         }
         const int idx = (ks * TM + i) * TN + j;
         if (idx % EVERY == EVERY - 1 && idx / EVERY < L) {
@@ -498,6 +507,7 @@ __device__ __forceinline__ void mma_ktile(const char* At, const char* Bt, int wr
         __builtin_amdgcn_sched_barrier(0);
       }
   }
+  f0 = f[0];
 }
 
 // C[rows_e, N] = A[rows_e, K] . op(B[e]) with B K-contiguous ([N,K]) or MN-contiguous ([K,N]).
@@ -664,12 +674,20 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
+    // k-tile 0 has landed once only younger operations are in flight: the younger k-tiles and
+    // the stores that the previous epilogue issued after its prefetch
+    wait_vm_le(min(NS - 2, nkt - 1) * L + st_after);
+    block_barrier();
+    Frags<TM, TN> f0;     // fragments of the first k-step of the coming k-tile, read one tile ahead
+    if (wave_has_rows)
+      load_frags<BK, TM, TN, true, B_KC, BM, BN>(f0, smem + cur * STAGE, smem + cur * STAGE + A_BYTES, wm * WTM, wn * WTN, 0, lane);
+
     for (int kt = 0; kt < nkt; ++kt) {
-      // k-tile kt has landed once only younger operations are in flight: the younger k-tiles
-      // and, before k-tile 0, the stores that the previous epilogue issued after its prefetch
-      if (kt == 0) wait_vm_le(min(NS - 2, nkt - 1) * L + st_after);
-      else wait_tiles<L, NS - 2>(min(NS - 2, nkt - 1 - kt));
-      block_barrier();   // everyone's part of tile kt is in LDS; everyone is done reading tile kt-1
+      // k-tile kt+1 has to be in LDS before this tile's MFMAs: its first fragments are read
+      // while they run, so that no wave waits for LDS behind the barrier of the next tile
+      if (kt == 0) wait_vm_le(max(min(NS - 1, nkt) - 2, 0) * L + st_after);
+      else wait_tiles<L, NS - 3>(min(NS - 3, nkt - 2 - kt));
+      block_barrier();   // everyone's part of tile kt+1 is in LDS; everyone is done reading tile kt-1
       if (kt == 0 && tid == 0)         // publish the unit after this one
         lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, ui.total));
       if (kt == 1) {                    // the box was written before this k-tile's barrier
@@ -680,9 +698,10 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
       issue_setup(kt + NS - 1, tgt);
       const bool do_issue = dbg_loads && kt + NS - 1 < nkt;
       const char* st = smem + cur * STAGE;
+      const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
       if (wave_has_rows && dbg_mma) {
-        mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, wm * WTM, wn * WTN, acc, do_issue,
-                                                     [&](int piece) { issue_piece(cur_u, piece); });
+        mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, kt + 1 < nkt, wm * WTM, wn * WTN,
+                                                     f0, acc, do_issue, [&](int piece) { issue_piece(cur_u, piece); });
       } else if (do_issue) {
 #pragma unroll
         for (int i = 0; i < L; ++i) issue_piece(cur_u, i);
@@ -1142,7 +1161,7 @@ int simt_ragged_k(const void* A, int64_t lda, const int32_t* a_map, const void* 
 #define PK_WG_SMALL 128, 128, 64, 2, 2, 3
 #define PK_WG_SMALL_THREADS 256
 
-#define PK_RM_ALT 128, 128, 64, 2, 2, 3      /* output widths that are a multiple of 128 but not of 256 */
+#define PK_RM_ALT 128, 128, 64, 2, 2, 4      /* output widths that are a multiple of 128 but not of 256 */
 bool mfma_shape_ok(int64_t H, int64_t I) { return H % 128 == 0 && I % 128 == 0; }
 
 // Pick the tile width by the output width N of the GEMM (for the gate/up kernel a tile holds
@@ -1156,8 +1175,10 @@ int launch_rm(mf::RaggedMParams& p, int64_t A, int64_t N, int kernel_id, hipStre
     // workgroup (then the last round of units runs on a half-empty chip)
     const int64_t big_units = (A / 256 + p.E / 2) * p.n_tiles;
     const bool lowm = big_units < (int64_t)PK_RM_LOWM_UNITS * mf::persistent_grid();
-    if (lowm) return mf::launch_ragged_m<PK_RM_LOWM, B_KC, EPI>(p, A, kernel_id, s);
-    return mf::launch_ragged_m<PK_RM_CFG, B_KC, EPI>(p, A, kernel_id, s);
+    // the scaled SwiGLU backward holds three packed outputs per chunk: with 256-row units it does
+    // not fit the register file (measured 2 % slower than 128-row units at 16,384 tokens)
+    if (lowm || EPI == mf::EPI_SWIGLU_BWD_SCALED) return mf::launch_ragged_m<PK_RM_LOWM, B_KC, EPI>(p, A, kernel_id, s);
+    if constexpr (EPI != mf::EPI_SWIGLU_BWD_SCALED) return mf::launch_ragged_m<PK_RM_CFG, B_KC, EPI>(p, A, kernel_id, s);
   }
   const int64_t per_tile_alt = (EPI == mf::EPI_SWIGLU) ? 64 : 128;
   p.n_tiles = (int32_t)(N / per_tile_alt);
