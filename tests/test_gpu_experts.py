@@ -197,6 +197,39 @@ def test_argument_errors(dev):
         ops.grouped_swiglu_fwd(z.float(), w, w2, w, starts)    # dtype mismatch
 
 
+def test_scaled_backward_argument_errors_and_empty_input(dev):
+    """Status codes of the C entry point itself: nothing is launched for a bad call."""
+    from piper_amd import _lib
+    from piper_amd._lib import PK_BF16, current_stream, ptr
+    lib = _lib.load()
+    E, H, I, T, K = 2, 256, 128, 16, 2
+    A = T * K
+    bf = dict(device=dev, dtype=torch.bfloat16)
+    d_out, w2 = torch.zeros(T, H, **bf), torch.zeros(E, H, I, **bf)
+    g, u, dg, du, hs = (torch.zeros(A, I, **bf) for _ in range(5))
+    perm = torch.arange(A, dtype=torch.int32, device=dev)
+    sc = torch.ones(T, K, device=dev)
+    ds = torch.zeros(T, K, device=dev)
+    starts = torch.tensor([0, A // 2, A], dtype=torch.int32, device=dev)
+    need = int(lib.pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes(A, I))
+    assert need == (I // 64) * A * 4
+    ws = torch.zeros(need // 4, device=dev)
+    s = current_stream(dev)
+
+    def call(ws_ptr, ws_bytes, rows=A, row_map=ptr(perm), div=K):
+        return lib.pk_grouped_swiglu_dgrad_dh_scaled(ptr(d_out), row_map, div, ptr(sc), ptr(w2), ptr(g), ptr(u), ptr(starts),
+                                                     ptr(dg), ptr(du), ptr(hs), ptr(ds), ws_ptr, ws_bytes, rows, H, I, E,
+                                                     PK_BF16, s)
+    assert call(ptr(ws), need) == 0
+    assert call(ptr(ws), need - 4) == -4          # PK_ERR_WORKSPACE
+    assert call(None, 0) == -4
+    assert call(ptr(ws), need, row_map=None) == -1     # PK_ERR_ARG: the gather map is not optional here
+    assert call(ptr(ws), need, div=0) == -1
+    assert call(None, 0, rows=0) == 0                  # no rows: nothing to do, nothing required
+    assert lib.pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes(-1, I) == -1
+    torch.cuda.synchronize()
+
+
 def test_grouped_gemms_replay_in_a_hip_graph(dev):
     """The persistent kernels take their work units from counters that the last workgroup of a
     launch resets: a captured graph must give the eager result on every replay, also with new
