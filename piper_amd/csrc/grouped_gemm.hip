@@ -384,12 +384,34 @@ __device__ __forceinline__ void sched_finish(SchedSlot* slot) {
   }
 }
 
+// Division of a non-negative int32 by a divisor fixed per launch without the ~25 instructions of
+// the general integer division: a shift for powers of two, otherwise multiply-high by
+// floor(2^(31+s)/d)+1 and shift by s-1 with s = ceil(log2 d) (exact for 0 <= n < 2^31).
+struct FastDiv {
+  uint32_t mul;    // 0: divisor is 2^shift
+  int32_t shift;
+};
+inline FastDiv make_fastdiv(int64_t d) {
+  FastDiv f = {0u, 0};
+  if (d <= 1) return f;
+  int s = 0;
+  while (((int64_t)1 << s) < d) ++s;
+  if (((int64_t)1 << s) == d) { f.shift = s; return f; }
+  f.mul = (uint32_t)((((uint64_t)1 << (31 + s)) / (uint64_t)d) + 1u);
+  f.shift = s - 1;
+  return f;
+}
+__device__ __forceinline__ int fastdiv(int n, const FastDiv f) {
+  const uint32_t u = (uint32_t)n;
+  return (int)((f.mul ? __umulhi(u, f.mul) : u) >> f.shift);
+}
+
 struct RaggedMParams {
   const bf16_t* A0;      // A operand of k-segment 0, row-major [rows, lda]
   const bf16_t* A1;      // k-segment 1 (nseg == 2)
   int64_t lda;
-  const int32_t* row_map;  // optional gather of A rows: src = row_map[row] / map_div
-  int32_t map_div;
+  const int32_t* row_map;  // optional gather of A rows: src = row_map[row] / divisor of map_div
+  FastDiv map_div;
   const bf16_t* B0;      // weights of k-segment 0 (EPI_SWIGLU: gate matrix)
   const bf16_t* B1;      // weights of k-segment 1 (EPI_SWIGLU: up matrix)
   int64_t ldb;
@@ -618,7 +640,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
           const int m = row_map[t.row0 + rr];
           if (lane / CPR == r) sel = m;
         }
-        src = sel / p.map_div;
+        src = fastdiv(sel, p.map_div);
       } else {
         src = t.row0 + min(rbase + lane / CPR, t.rows - 1);
       }
@@ -855,7 +877,7 @@ struct WgradParams {
   const int32_t* starts;
   const int32_t* order;      // optional [E]: experts by descending row count
   int32_t E;
-  int32_t map_div;
+  FastDiv map_div;
   int32_t accumulate;
   int32_t tiles_per_expert;  // (M/BM)*(N/BN), identical for the three problems
   int32_t nprob;
@@ -910,13 +932,34 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
   const bf16_t* const Abase = q.A + (int64_t)mt * BM;
   const bf16_t* const Bbase = q.B + (int64_t)nt * BN;
   const int64_t lda = q.lda, ldb = q.ldb;
-  const int map_div = p.map_div;
+  const FastDiv map_div = p.map_div;
 
-  auto issue = [&](int kt, int stage) {
+  // Source rows of the k-tile that is issued next (wave-uniform, -1 past the expert's end).  They
+  // are fetched one tile ahead, so the scalar loads of the row map run under the previous tile's
+  // MFMAs instead of in front of the loads.
+  constexpr int NA = LA * A_RPI, NB = LB * B_RPI;
+  int arow[NA], brow[NB];
+  auto fetch_rows = [&](int kt) {
+    const int k0 = row_begin + kt * BK;
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      const int row = k0 + wave * NA + i;     // piece i / A_RPI of this wave, row i % A_RPI of the piece
+      int v = -1;
+      if (row < row_end) v = a_map ? fastdiv(a_map[row], map_div) : row;
+      arow[i] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int row = k0 + wave * NB + i;
+      int v = -1;
+      if (row < row_end) v = b_map ? fastdiv(b_map[row], map_div) : row;
+      brow[i] = v;
+    }
+  };
+  auto issue = [&](int stage) {
     char* st = smem + stage * STAGE;
     const uint32_t a_lds = lds_addr(st) + (wave * LA) * 1024;
     const uint32_t b_lds = lds_addr(st + A_BYTES) + (wave * LB) * 1024;
-    const int k0 = row_begin + kt * BK;
 #pragma unroll
     for (int i = 0; i < LA; ++i) {
       int krow, cofs;
@@ -924,11 +967,9 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
       const void* src = g_zero16;
 #pragma unroll
       for (int r = 0; r < A_RPI; ++r) {
-        const int row = k0 + (wave * LA + i) * A_RPI + r;     // wave-uniform
-        if (row < row_end) {
-          int64_t rr = row;
-          if (a_map) rr = a_map[row] / map_div;
-          const bf16_t* cand = Abase + rr * lda;
+        const int v = arow[i * A_RPI + r];
+        if (v >= 0) {
+          const bf16_t* cand = Abase + (int64_t)v * lda;
           if (lane / A_CPR == r) src = cand + cofs;
         }
       }
@@ -941,11 +982,9 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
       const void* src = g_zero16;
 #pragma unroll
       for (int r = 0; r < B_RPI; ++r) {
-        const int row = k0 + (wave * LB + i) * B_RPI + r;
-        if (row < row_end) {
-          int64_t rr = row;
-          if (b_map) rr = b_map[row] / map_div;
-          const bf16_t* cand = Bbase + rr * ldb;
+        const int v = brow[i * B_RPI + r];
+        if (v >= 0) {
+          const bf16_t* cand = Bbase + (int64_t)v * ldb;
           if (lane / B_CPR == r) src = cand + cofs;
         }
       }
@@ -963,7 +1002,11 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
 
 #pragma unroll
   for (int s = 0; s < NS - 1; ++s)
-    if (s < nkt) issue(s, s);
+    if (s < nkt) {
+      fetch_rows(s);
+      issue(s);
+    }
+  if (NS - 1 < nkt) fetch_rows(NS - 1);
   int cur = 0, nxt = NS - 1;
   for (int kt = 0; kt < nkt; ++kt) {
     if (kt + NS - 2 < nkt) wait_dma<(NS - 2) * (LA + LB)>(); else wait_dma<0>();
@@ -971,7 +1014,8 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
 #ifdef PK_GEMM_DEBUG
     if (!(p.debug & 2))
 #endif
-    if (kt + NS - 1 < nkt) issue(kt + NS - 1, nxt);
+    if (kt + NS - 1 < nkt) issue(nxt);
+    if (kt + NS < nkt) fetch_rows(kt + NS);
     const char* st = smem + cur * STAGE;
 #ifdef PK_GEMM_DEBUG
     if (!(p.debug & 1))
@@ -1247,7 +1291,7 @@ int pk_grouped_swiglu_fwd(const void* x_rows, const int32_t* row_map, int64_t ro
   if (rc) return rc;
   if (A == 0) return PK_OK;
   if (!x_rows || !w1 || !w2 || !w3 || !starts || !g || !u || !h || !y) return PK_ERR_ARG;
-  if (row_map && row_map_div <= 0) return PK_ERR_ARG;
+  if (row_map && (row_map_div <= 0 || row_map_div > 0x7fffffffll)) return PK_ERR_ARG;
   if (!row_map) row_map_div = 1;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PK_F32)
@@ -1257,7 +1301,7 @@ int pk_grouped_swiglu_fwd(const void* x_rows, const int32_t* row_map, int64_t ro
 
   mf::RaggedMParams p = {};
   p.A0 = (const bf16_t*)x_rows; p.A1 = nullptr; p.lda = H;
-  p.row_map = row_map; p.map_div = (int32_t)row_map_div;
+  p.row_map = row_map; p.map_div = mf::make_fastdiv(row_map_div);
   p.B0 = (const bf16_t*)w1; p.B1 = (const bf16_t*)w3; p.ldb = H; p.strideB = I * H;
   p.starts = starts; p.E = (int32_t)E; p.Kseg = (int32_t)H; p.nseg = 1;
   p.O0 = (bf16_t*)g; p.O1 = (bf16_t*)u; p.O2 = (bf16_t*)h; p.ldc = I;
@@ -1321,7 +1365,7 @@ int pk_grouped_swiglu_dgrad_dh_scaled(const void* d_out, const int32_t* row_map,
   int rc = check_common(A, H, I, E, dtype);
   if (rc) return rc;
   if (A == 0) return PK_OK;
-  if (!d_out || !row_map || row_map_div <= 0 || !scores || !w2 || !g || !u || !starts || !d_g || !d_u || !hs || !d_scores)
+  if (!d_out || !row_map || row_map_div <= 0 || row_map_div > 0x7fffffffll || !scores || !w2 || !g || !u || !starts || !d_g || !d_u || !hs || !d_scores)
     return PK_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   const bool simt = dtype == PK_F32 || !mfma_shape_ok(H, I) || !all_aligned16({d_out, w2, g, u, d_g, d_u, hs});
@@ -1344,7 +1388,7 @@ int pk_grouped_swiglu_dgrad_dh_scaled(const void* d_out, const int32_t* row_map,
   if (!workspace || workspace_bytes < need) return PK_ERR_WORKSPACE;
   mf::RaggedMParams p = {};
   p.A0 = (const bf16_t*)d_out; p.lda = H;
-  p.row_map = row_map; p.map_div = (int32_t)row_map_div;
+  p.row_map = row_map; p.map_div = mf::make_fastdiv(row_map_div);
   p.B0 = (const bf16_t*)w2; p.ldb = I; p.strideB = H * I;
   p.starts = starts; p.E = (int32_t)E; p.Kseg = (int32_t)H; p.nseg = 1;
   p.Gin = (const bf16_t*)g; p.Uin = (const bf16_t*)u;
@@ -1409,7 +1453,7 @@ static int wgrad_impl(const void* d_y, int dy_gathered, const void* h, const voi
   if (d_w2 && A > 0 && (!d_y || !h)) return PK_ERR_ARG;
   if (d_w1 && A > 0 && (!d_g || !x_rows)) return PK_ERR_ARG;
   if (d_w3 && A > 0 && (!d_u || !x_rows)) return PK_ERR_ARG;
-  if (row_map && row_map_div <= 0) return PK_ERR_ARG;
+  if (row_map && (row_map_div <= 0 || row_map_div > 0x7fffffffll)) return PK_ERR_ARG;
   if (dy_gathered && !row_map) return PK_ERR_ARG;
   if (!row_map) row_map_div = 1;
   const int32_t* dy_map = dy_gathered ? row_map : nullptr;
@@ -1440,7 +1484,7 @@ static int wgrad_impl(const void* d_y, int dy_gathered, const void* h, const voi
     q.C = (bf16_t*)d_w3; q.M = (int32_t)I; q.N = (int32_t)H;
   }
   if (n == 0) return PK_OK;
-  p.starts = starts; p.order = expert_order; p.E = (int32_t)E; p.map_div = (int32_t)row_map_div;
+  p.starts = starts; p.order = expert_order; p.E = (int32_t)E; p.map_div = mf::make_fastdiv(row_map_div);
   p.accumulate = accumulate ? 1 : 0;
 #ifdef PK_GEMM_DEBUG
   { const char* d = getenv("PK_GEMM_DEBUG_MODE"); p.debug = d ? atoi(d) : 0; }
