@@ -125,13 +125,32 @@ def _queue_expert_wgrad(params, d_y, h, d_g, d_u, x, starts, perm, top_k, order,
     _WGRAD_QUEUE.push(run)
 
 
+def _traced_without_data(*tensors) -> bool:
+    """True under fake-tensor propagation (Dynamo, make_fx) or on the meta device: the call is only
+    asked for the output's shape, dtype and whether it takes part in autograd."""
+    from torch._subclasses.fake_tensor import FakeTensor
+    return any(t.is_meta or isinstance(t, FakeTensor) for t in tensors)
+
+
+def _bmm_experts_shape_only(w1, w2, w3, x):
+    out = torch.empty_like(x)
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (w1, w2, w3, x)):
+        out.requires_grad_(True)
+    return out
+
+
 def _bmm_experts_autograd(w1, w2, w3, x, num_tokens_per_expert):
-    if x.is_meta:
-        return torch.empty_like(x)
+    # The reference binds one traceable Python function to every dispatch key, the Autograd key
+    # included (qwen3_bmm_experts_patch.py:67-75), so Dynamo's fake-tensor propagation runs this
+    # kernel too: it must not touch device pointers then.
+    if _traced_without_data(w1, w2, w3, x, num_tokens_per_expert):
+        return _bmm_experts_shape_only(w1, w2, w3, x)
     return _BmmExpertsFn.apply(w1, w2, w3, x, num_tokens_per_expert)
 
 
 def _bmm_experts_forward_only(w1, w2, w3, x, num_tokens_per_expert):
+    if _traced_without_data(w1, w2, w3, x, num_tokens_per_expert):
+        return torch.empty_like(x)
     starts = ops.counts_to_starts(num_tokens_per_expert)
     return ops.grouped_swiglu_fwd(x, w1, w2, w3, starts)[0]
 
@@ -349,11 +368,71 @@ class _ExpertRegionFn(torch.autograd.Function):
         return d_x, d_wg, d_b, d_w1, d_w2, d_w3, None, None, None, (d_out if need[9] else None)
 
 
+# The fused region and the RMSNorm are torch.library operators too (namespace piper_amd), for the same
+# reason the reference wraps its expert segment in one (qwen3_bmm_experts_patch.py:56-75): the model
+# is captured by Dynamo with fullgraph=True (src/compile.py:273), which cannot look inside a
+# function that launches kernels through a C ABI.  As graph nodes they are opaque calls whose
+# output shape comes from the fake-tensor branch of their kernels.
+_REGION_LIBS = []
+
+
+def _expert_region_autograd(x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale, residual):
+    ts = [t for t in (x, w_gate, gate_bias, w1, w2, w3, residual) if t is not None]
+    if _traced_without_data(*ts):
+        out = torch.empty_like(x)
+        if torch.is_grad_enabled() and any(t.requires_grad for t in ts):
+            out.requires_grad_(True)
+        return out
+    return _ExpertRegionFn.apply(x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale, residual)
+
+
+def _expert_region_forward_only(x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale, residual):
+    with torch.no_grad():
+        return _expert_region_autograd(x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale, residual)
+
+
+def _rmsnorm_autograd(x, weight, eps):
+    if _traced_without_data(x, weight):
+        out = torch.empty_like(x)
+        if torch.is_grad_enabled() and (x.requires_grad or weight.requires_grad):
+            out.requires_grad_(True)
+        return out
+    return _RMSNormFn.apply(x, weight, eps)
+
+
+def _rmsnorm_forward_only(x, weight, eps):
+    with torch.no_grad():
+        return _rmsnorm_autograd(x, weight, eps)
+
+
+def register_region_ops() -> bool:
+    """Define ``piper_amd::expert_region`` and ``piper_amd::rmsnorm`` (done when this module is
+    imported: a registration cannot happen inside a function Dynamo is tracing).  Returns True when
+    this call registered them."""
+    if _REGION_LIBS:
+        return False
+    lib = torch.library.Library("piper_amd", "DEF")
+    lib.define("expert_region(Tensor x, Tensor w_gate, Tensor? gate_bias, Tensor w1, Tensor w2, Tensor w3, "
+               "int top_k, bool route_norm, float route_scale, Tensor? residual) -> Tensor")
+    lib.define("rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor")
+    for name, fwd, auto in (("expert_region", _expert_region_forward_only, _expert_region_autograd),
+                            ("rmsnorm", _rmsnorm_forward_only, _rmsnorm_autograd)):
+        lib.impl(name, fwd, "CUDA")
+        lib.impl(name, auto, "AutogradCUDA")
+        lib.impl(name, fwd, "Meta")
+        # CPU tensors reach the kernels' own check and are refused there; fake CPU tensors get a shape
+        lib.impl(name, fwd, "CPU")
+        lib.impl(name, auto, "AutogradCPU")
+    _REGION_LIBS.append(lib)
+    return True
+
+
 def expert_region(x, w_gate, gate_bias, w1, w2, w3, *, top_k: int, route_norm: bool, route_scale: float = 1.0,
                   residual=None):
     """The whole MoE expert region of AnnotatedMoE.forward (qwen3.py:233-289) on x [T,H].
     `residual` [T,H] is added to the result in the combine kernel."""
-    return _ExpertRegionFn.apply(x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale, residual)
+    return torch.ops.piper_amd.expert_region(x, w_gate, gate_bias, w1, w2, w3, int(top_k), bool(route_norm),
+                                             float(route_scale), residual)
 
 
 class _RMSNormFn(torch.autograd.Function):
@@ -373,7 +452,7 @@ class _RMSNormFn(torch.autograd.Function):
 def rmsnorm(x, weight, eps: float = 1e-6):
     """RMSNorm over the last dimension (the block's ffn_norm, qwen3.py:313-314)."""
     shape = x.shape
-    return _RMSNormFn.apply(x.reshape(-1, shape[-1]), weight, eps).reshape(shape)
+    return torch.ops.piper_amd.rmsnorm(x.reshape(-1, shape[-1]), weight, float(eps)).reshape(shape)
 
 
 def moe_block(h, norm_weight, w_gate, gate_bias, w1, w2, w3, *, top_k: int, route_norm: bool,
@@ -382,3 +461,6 @@ def moe_block(h, norm_weight, w_gate, gate_bias, w1, w2, w3, *, top_k: int, rout
     added in the combine kernel."""
     return expert_region(rmsnorm(h, norm_weight, norm_eps), w_gate, gate_bias, w1, w2, w3, top_k=top_k,
                          route_norm=route_norm, route_scale=route_scale, residual=h)
+
+
+register_region_ops()

@@ -197,6 +197,30 @@ def test_argument_errors(dev):
         ops.grouped_swiglu_fwd(z.float(), w, w2, w, starts)    # dtype mismatch
 
 
+def test_reference_operator_under_dynamo_fullgraph(dev):
+    """The op traced by Dynamo with fullgraph=True (src/compile.py:273) and run by the eager
+    backend gives the same forward and gradients as the direct call."""
+    counts = [5, 0, 130, 61]
+    x, w1, w2, w3, dy, cnt = _make(9, counts, 256, 128, torch.bfloat16)
+    X, W1, W2, W3, DY, CNT = (t.to(dev) for t in (x, w1, w2, w3, dy, cnt))
+
+    def region(w1, w2, w3, x, c):
+        return F_.bmm_experts(w1, w2, w3, x, c)
+
+    def run(fn):
+        leaves = [t.clone().requires_grad_(True) for t in (W1, W2, W3, X)]
+        out = fn(*leaves, CNT)
+        grads = torch.autograd.grad(out, leaves, DY)
+        return out, grads
+
+    torch._dynamo.reset()
+    o1, g1 = run(region)
+    o2, g2 = run(torch.compile(region, backend="eager", fullgraph=True))
+    assert torch.equal(o1, o2)
+    for a, b in zip(g1, g2):
+        assert torch.equal(a, b)
+
+
 def test_scaled_backward_argument_errors_and_empty_input(dev):
     """Status codes of the C entry point itself: nothing is launched for a bad call."""
     from piper_amd import _lib

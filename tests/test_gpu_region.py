@@ -155,6 +155,32 @@ def test_fused_and_piecewise_paths_agree(dev):
         assert rel_err(g1[k], g2[k]) <= 1e-2, k
 
 
+def test_block_captured_by_dynamo_fullgraph_matches_eager(dev):
+    """MoEFeedForwardBlock (ffn_norm -> experts -> residual) under torch.compile(fullgraph=True),
+    as the reference captures its model (src/compile.py:273): identical forward and gradients."""
+    from piper_amd.moe import MoEFeedForwardBlock
+    args = MoEArgs(num_experts=8, top_k=2, route_norm=True)
+    torch.manual_seed(1)
+    blk = MoEFeedForwardBlock(args, dim=256, hidden_dim=128, dtype=torch.bfloat16).to(dev)
+    blk.moe.init_weights()
+    x = torch.randn(2, 64, 256, device=dev, dtype=torch.bfloat16)
+    d = torch.randn_like(x)
+
+    def run(fn):
+        blk.zero_grad(set_to_none=True)
+        xi = x.clone().requires_grad_(True)
+        y = fn(xi)
+        y.backward(d)
+        return y.detach(), xi.grad, {n: p.grad.clone() for n, p in blk.named_parameters()}
+
+    torch._dynamo.reset()
+    y1, dx1, g1 = run(blk)
+    y2, dx2, g2 = run(torch.compile(blk, backend="eager", fullgraph=True))
+    assert torch.equal(y1, y2) and torch.equal(dx1, dx2)
+    for n in g1:
+        assert torch.equal(g1[n], g2[n]), n
+
+
 def test_module_mirrors_reference_layer(dev):
     """AnnotatedMoE with the reference's parameter names runs both data flows."""
     args = MoEArgs(num_experts=8, top_k=2, route_norm=True)
