@@ -132,6 +132,38 @@ def test_bf16_region_against_fp32_oracle(dev, cfg, fused):
         assert int((aux["counts"] == 0).sum()) > 0, "this case is meant to contain empty experts"
 
 
+ODD_SHAPES = [
+    # name, T, H, E, K, I, dtype, route_norm, zipf  -- expert counts that are not a power of two, top-1,
+    # fewer rows than one wave, widths on every GEMM path (256-wide, 128-wide, generic FMA kernel)
+    ("top1-e5", 37, 128, 5, 1, 128, torch.bfloat16, False, None),
+    ("k3-e130", 200, 384, 130, 3, 256, torch.bfloat16, True, None),
+    ("one-token", 1, 256, 8, 2, 128, torch.bfloat16, True, None),
+    ("k8-of-8", 65, 256, 8, 8, 384, torch.bfloat16, True, None),
+    ("narrow", 90, 96, 6, 2, 80, torch.bfloat16, True, None),
+    ("f32-k3", 77, 128, 7, 3, 64, torch.float32, True, 1.2),
+    ("skewed", 700, 512, 40, 4, 256, torch.bfloat16, True, 1.2),
+]
+
+
+@pytest.mark.parametrize("name,T,H,E,K,I,dtype,route_norm,zipf", ODD_SHAPES, ids=[c[0] for c in ODD_SHAPES])
+def test_region_on_odd_shapes(dev, name, T, H, E, K, I, dtype, route_norm, zipf):
+    print(f"[case] region odd shape {name}", flush=True)
+    cfg = ExpertRegionConfig(name, tokens=T, hidden=H, num_experts=E, top_k=K, inter=I, dtype=dtype,
+                             route_norm=route_norm, zipf_s=zipf, zipf_alpha=1.5 if zipf else 0.0)
+    inp = make_expert_region_inputs(cfg)
+    out_ref, aux, g_ref = _oracle_fwd_bwd(inp, cfg, compute_dtype=torch.float32)
+    out, g = _gpu_fwd_bwd(inp, cfg, dev, fused=True)
+    tol = BF16_TOL if dtype == torch.bfloat16 else F32_TOL
+    assert out.dtype == dtype and rel_err(out, out_ref) <= tol
+    for k in g_ref:
+        assert rel_err(g[k], g_ref[k]) <= tol, k
+    # and the op-by-op path on the same inputs
+    out2, g2 = _gpu_fwd_bwd(inp, cfg, dev, fused=False)
+    assert torch.equal(out, out2)
+    for k in g_ref:
+        assert rel_err(g2[k], g_ref[k]) <= tol, k
+
+
 def test_wgrad_on_side_stream_gives_identical_results(dev):
     inp = make_expert_region_inputs(SMALL_BF16)
     o1, g1 = _gpu_fwd_bwd(inp, SMALL_BF16, dev, fused=True)
