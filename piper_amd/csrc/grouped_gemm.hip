@@ -487,10 +487,13 @@ struct Stage32 {
 // the MFMAs as well, which keeps the LDS queue short while the ring is being written.  Operands are passed to the MFMA
 // swapped (B first) so that a lane's accumulator holds 4 CONSECUTIVE columns of ONE row:
 //   acc[i][j][v] = C[row = 32*i + lane%32][col = 32*j + 8*(v/4) + 4*(lane/32) + v%4]
+// There is no branch between the MFMAs: the L loads are issued for every k-tile (the caller
+// points them at a block of zeros when no tile is left to fetch) and the first fragments of the
+// "next tile" are always read (the caller passes any tile of the ring when there is none).
 template <int BK, int TM, int TN, bool A_KC, bool B_KC, int ACOLS, int BCOLS, int L, typename F>
 __device__ __forceinline__ void mma_ktile(const char* At, const char* Bt, const char* At_next, const char* Bt_next,
-                                          bool has_next_tile, int wrow0, int wcol0, Frags<TM, TN>& f0,
-                                          floatx16_t (&acc)[TM][TN], bool do_issue, F&& issue_one) {
+                                          int wrow0, int wcol0, Frags<TM, TN>& f0,
+                                          floatx16_t (&acc)[TM][TN], F&& issue_one) {
   const int lane = threadIdx.x & 63;
   constexpr int KS = BK / 16, NM = KS * TM * TN;
   constexpr int EVERY = NM / L > 0 ? NM / L : 1;
@@ -518,17 +521,13 @@ __device__ __forceinline__ void mma_ktile(const char* At, const char* Bt, const 
         // k-step starts with row 0) and at most one load behind each MFMA
         __builtin_amdgcn_sched_barrier(0);
         const int m = i * TN + j;
-        if (!last || has_next_tile) {
-          if (m < TN)
-            f[(ks + 1) & 1].b[m] = B_KC ? frag_kc<BK>(Bn, wcol0 + 32 * m, ksn, lane) : frag_mn<BCOLS>(Bn, wcol0 + 32 * m, ksn, lane);
-          else if (m < TN + TM)
-            f[(ks + 1) & 1].a[m - TN] = A_KC ? frag_kc<BK>(An, wrow0 + 32 * (m - TN), ksn, lane)
-                                             : frag_mn<ACOLS>(An, wrow0 + 32 * (m - TN), ksn, lane);
-        }
+        if (m < TN)
+          f[(ks + 1) & 1].b[m] = B_KC ? frag_kc<BK>(Bn, wcol0 + 32 * m, ksn, lane) : frag_mn<BCOLS>(Bn, wcol0 + 32 * m, ksn, lane);
+        else if (m < TN + TM)
+          f[(ks + 1) & 1].a[m - TN] = A_KC ? frag_kc<BK>(An, wrow0 + 32 * (m - TN), ksn, lane)
+                                           : frag_mn<ACOLS>(An, wrow0 + 32 * (m - TN), ksn, lane);
         const int idx = (ks * TM + i) * TN + j;
-        if (idx % EVERY == EVERY - 1 && idx / EVERY < L) {
-          if (do_issue) issue_one(idx / EVERY);
-        }
+        if (idx % EVERY == EVERY - 1 && idx / EVERY < L) issue_one(idx / EVERY);
         __builtin_amdgcn_sched_barrier(0);
       }
   }
@@ -648,6 +647,11 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     }
   };
 
+#ifdef PK_GEMM_DEBUG
+  const bool dbg_loads_v = !(p.debug & 2), dbg_mma = !(p.debug & 1);
+#else
+  constexpr bool dbg_loads_v = true, dbg_mma = true;
+#endif
   // DMA of k-tile `kt` of unit `t` into ring stage `stage`: piece 0..LA-1 = A, LA..L-1 = B
   int is_k0 = 0, is_seg = 0;
   uint32_t is_a = 0, is_b = 0;
@@ -657,26 +661,28 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     is_a = lds_addr(smem + stage * STAGE) + (wave * LA) * 1024;
     is_b = lds_addr(smem + stage * STAGE + A_BYTES) + (wave * LB) * 1024;
   };
+  // Every k-tile slot of the loop issues its L loads, so the count of loads in flight does not
+  // depend on where in a unit the loop is: with `real` false (no tile left to fetch) they read a
+  // block of zeros into the stage, which nobody reads before it is filled again.
+  bool is_real = true;
   auto issue_piece = [&](const Unit& t, int piece) {
     if (piece < LA) {
       const bf16_t* A = is_seg ? p.A1 : p.A0;
-      dma16(A + t.a_off[piece] + is_k0, is_a + piece * 1024);
+      const void* src = A + t.a_off[piece] + is_k0;
+      dma16(is_real ? src : (const void*)g_zero16, is_a + piece * 1024);
     } else {
       const int i = piece - LA;
       const bf16_t* B = (EPI == EPI_SWIGLU) ? (b_mat[i] ? p.B1 : p.B0) : (is_seg ? p.B1 : p.B0);
-      dma16(B + t.b_base + b_loff[i] + (B_KC ? (int64_t)is_k0 : (int64_t)is_k0 * p.ldb), is_b + i * 1024);
+      const void* src = B + t.b_base + b_loff[i] + (B_KC ? (int64_t)is_k0 : (int64_t)is_k0 * p.ldb);
+      dma16(is_real ? src : (const void*)g_zero16, is_b + i * 1024);
     }
   };
   auto issue_tile = [&](const Unit& t, int kt, int stage) {
     issue_setup(kt, stage);
+    is_real = dbg_loads_v && kt < nkt;
 #pragma unroll
     for (int i = 0; i < L; ++i) issue_piece(t, i);
   };
-#ifdef PK_GEMM_DEBUG
-  const bool dbg_loads = !(p.debug & 2), dbg_mma = !(p.debug & 1);
-#else
-  constexpr bool dbg_loads = true, dbg_mma = true;
-#endif
 
   int st_after = 0;     // stores this wave issued after its latest prefetch
   Unit cur_u, nxt_u;
@@ -684,8 +690,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   nxt_u = cur_u;
   int cur = 0;          // ring stage of k-tile 0 of the current unit
 #pragma unroll
-  for (int s = 0; s < NS - 1; ++s)
-    if (s < nkt && dbg_loads) issue_tile(cur_u, s, s);
+  for (int s = 0; s < NS - 1; ++s) issue_tile(cur_u, s, s);
 
   for (;;) {
     int unit_next = -1;
@@ -701,7 +706,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
 
     // k-tile 0 has landed once only younger operations are in flight: the younger k-tiles and
     // the stores that the previous epilogue issued after its prefetch
-    wait_vm_le(min(NS - 2, nkt - 1) * L + st_after);
+    wait_vm_le((NS - 2) * L + st_after);
     block_barrier();
     Frags<TM, TN> f0;     // fragments of the first k-step of the coming k-tile, read one tile ahead
     if (wave_has_rows)
@@ -710,8 +715,9 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     for (int kt = 0; kt < nkt; ++kt) {
       // k-tile kt+1 has to be in LDS before this tile's MFMAs: its first fragments are read
       // while they run, so that no wave waits for LDS behind the barrier of the next tile
-      if (kt == 0) wait_vm_le(max(min(NS - 1, nkt) - 2, 0) * L + st_after);
-      else wait_tiles<L, NS - 3>(min(NS - 3, nkt - 2 - kt));
+      // (NS-1+kt tiles have been requested, real or not; all but the NS-3 youngest must be there)
+      if (kt == 0) wait_vm_le((NS - 3) * L + st_after);
+      else wait_dma<(NS - 3) * L>();
       block_barrier();   // everyone's part of tile kt+1 is in LDS; everyone is done reading tile kt-1
       if (kt == 0 && tid == 0)         // publish the unit after this one
         lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, ui.total));
@@ -721,13 +727,13 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
       }
       const int tgt = cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1;   // stage of k-tile kt-1 = kt+NS-1
       issue_setup(kt + NS - 1, tgt);
-      const bool do_issue = dbg_loads && kt + NS - 1 < nkt;
+      is_real = dbg_loads_v && kt + NS - 1 < nkt;
       const char* st = smem + cur * STAGE;
       const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
       if (wave_has_rows && dbg_mma) {
-        mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, kt + 1 < nkt, wm * WTM, wn * WTN,
-                                                     f0, acc, do_issue, [&](int piece) { issue_piece(cur_u, piece); });
-      } else if (do_issue) {
+        mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN,
+                                                     f0, acc, [&](int piece) { issue_piece(cur_u, piece); });
+      } else {
 #pragma unroll
         for (int i = 0; i < L; ++i) issue_piece(cur_u, i);
       }
@@ -743,8 +749,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
       st_after = 0;
       if (has_next) {
 #pragma unroll
-        for (int s = 0; s < NS - 1; ++s)
-          if (s < nkt && dbg_loads) issue_tile(nxt_u, s, cur + s >= NS ? cur + s - NS : cur + s);
+        for (int s = 0; s < NS - 1; ++s) issue_tile(nxt_u, s, cur + s >= NS ? cur + s - NS : cur + s);
       }
     };
     if (!BWD) prefetch_next();
@@ -862,6 +867,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     unit = unit_next;
     par ^= 1;
   }
+  wait_dma<0>();   // the zero loads of the last k-tiles must not land in LDS that a later workgroup owns
   if (tid == 0) sched_finish(p.sched);
 }
 
@@ -957,6 +963,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
     }
   };
   uint32_t is_a = 0, is_b = 0;     // LDS destinations of this wave's pieces in the stage being filled
+  bool is_real = true;             // false: no tile left, the pieces read zeros (rows are not looked up)
   auto issue_setup = [&](int stage) {
     char* st = smem + stage * STAGE;
     is_a = lds_addr(st) + (wave * LA) * 1024;
@@ -972,7 +979,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
 #pragma unroll
       for (int r = 0; r < A_RPI; ++r) {
         const int v = arow[i * A_RPI + r];
-        if (v >= 0) {
+        if (is_real && v >= 0) {
           const bf16_t* cand = Abase + (int64_t)v * lda;
           if (lane / A_CPR == r) src = cand + cofs;
         }
@@ -986,7 +993,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
 #pragma unroll
       for (int r = 0; r < B_RPI; ++r) {
         const int v = brow[i * B_RPI + r];
-        if (v >= 0) {
+        if (is_real && v >= 0) {
           const bf16_t* cand = Bbase + (int64_t)v * ldb;
           if (lane / B_CPR == r) src = cand + cofs;
         }
@@ -1008,36 +1015,49 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
+  if constexpr (NS >= 3) {
+    // every slot issues its loads (rows past the expert's end read a block of zeros), so the
+    // number of loads in flight is the same at every k-tile
 #pragma unroll
-  for (int s = 0; s < NS - 1; ++s)
-    if (s < nkt) {
-      fetch_rows(s);
+    for (int s = 0; s < NS - 1; ++s) {
+      is_real = s < nkt;
+      if (is_real) fetch_rows(s);
       issue(s);
     }
-  if (NS - 1 < nkt) fetch_rows(NS - 1);
+    if (NS - 1 < nkt) fetch_rows(NS - 1);
+  } else {
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s)
+      if (s < nkt) {
+        fetch_rows(s);
+        issue(s);
+      }
+    if (NS - 1 < nkt) fetch_rows(NS - 1);
+  }
   int cur = 0, nxt = NS - 1;
   if constexpr (NS >= 3) {
     // Rings of three or more stages: the loads of tile kt+NS-1 and the fragment reads of the
     // next k-step are spread between the MFMAs, and the first fragments of tile kt+1 are read
     // during tile kt (the barrier at the top of tile kt waits for tile kt+1).
     constexpr int L = LA + LB;
-    wait_tiles<L, NS - 2>(min(NS - 2, nkt - 1));
+    wait_dma<(NS - 2) * L>();
     block_barrier();
     Frags<TM, TN> f0;
     load_frags<BK, TM, TN, false, false, BM, BN>(f0, smem, smem + A_BYTES, wm * WTM, wn * WTN, 0, lane);
     for (int kt = 0; kt < nkt; ++kt) {
-      wait_tiles<L, NS - 3>(min(NS - 3, nkt - 2 - kt));
+      wait_dma<(NS - 3) * L>();
       block_barrier();
-      const bool do_issue = kt + NS - 1 < nkt;
       issue_setup(nxt);
+      is_real = kt + NS - 1 < nkt;
       const char* st = smem + cur * STAGE;
       const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
-      mma_ktile<BK, TM, TN, false, false, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, kt + 1 < nkt, wm * WTM, wn * WTN,
-                                                     f0, acc, do_issue, [&](int piece) { issue_piece(piece); });
+      mma_ktile<BK, TM, TN, false, false, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN,
+                                                     f0, acc, [&](int piece) { issue_piece(piece); });
       if (kt + NS < nkt) fetch_rows(kt + NS);
       cur = cur + 1 == NS ? 0 : cur + 1;
       nxt = nxt + 1 == NS ? 0 : nxt + 1;
     }
+    wait_dma<0>();   // zero loads of the last k-tiles: the staging below reuses the ring
   } else {
     for (int kt = 0; kt < nkt; ++kt) {
       if (kt + NS - 2 < nkt) wait_dma<(NS - 2) * (LA + LB)>(); else wait_dma<0>();
