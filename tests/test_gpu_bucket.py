@@ -170,3 +170,37 @@ def test_cfg2_full_size_properties(dev):
     # padding elements have g == 0 -> update 0/(0+eps) = 0, also covered by the closed form
     assert (master.double() - expect).abs().max().item() <= ADAMW_TOL
     assert torch.equal(shadow, master.bfloat16())
+
+
+def test_timing_select_brackets_one_kernel_only(dev):
+    """pk_timing_select restricts the per-launch event pairs to one kernel id."""
+    from piper_amd import _lib
+    n = 1 << 16
+    g = (torch.randn(n, device=dev) * 1e-3).bfloat16()
+    flat = torch.zeros(n, device=dev)
+    p = torch.randn(n, device=dev)
+    m, v = torch.zeros_like(p), torch.zeros_like(p)
+
+    def work():
+        ops.bucket_pack([g], [0], flat, accumulate=False)
+        ops.adamw_fused(p, m, v, flat, step=1, lr=1e-3, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+
+    try:
+        _lib.timing_enable(True)
+        _lib.timing_collect()
+        work()
+        assert sorted(k for k, _ in _lib.timing_collect()) == ["adamw", "bucket_pack"]
+        _lib.timing_select("adamw")
+        work()
+        work()
+        rec = _lib.timing_collect()
+        assert [k for k, _ in rec] == ["adamw", "adamw"] and all(ms > 0 for _, ms in rec)
+        _lib.timing_select(None)
+        work()
+        assert len(_lib.timing_collect()) == 2
+        with pytest.raises(ValueError):
+            _lib.timing_select("no_such_kernel")
+    finally:
+        _lib.timing_select(None)
+        _lib.timing_enable(False)
+        _lib.timing_collect()
