@@ -138,6 +138,13 @@ PK_API int pk_combine_bwd(const void* d_out, const void* y_sorted, int dtype, co
                    const float* top_scores, void* d_y_sorted, float* d_top_scores, int64_t A,
                    int64_t H, int64_t K, pk_stream_t stream);
 
+/* buf[r, 0:width] = 0 for r in [*first_row, rows); first_row is a DEVICE pointer (for example
+ * starts + E, so nothing is read back).  The reference's bmm_experts returns zeros in the rows of
+ * its input that no expert owns (`out = x.new_zeros(...)`, qwen3_bmm_experts_patch.py:43), which
+ * the grouped kernels never touch. */
+PK_API int pk_zero_rows_from(void* buf, int dtype, const int32_t* first_row, int64_t rows, int64_t width,
+                      pk_stream_t stream);
+
 /* ------------------------------------------------------ RMSNorm in front of the region
  * The block's ffn_norm (qwen3.py:313-314; torchtitan builds it as RMSNorm(dim, eps=norm_eps),
  * eps 1e-6 in the Qwen3 configs, qwen3.py:28): y = x * rsqrt(mean_h(x^2) + eps) * weight, computed
@@ -162,7 +169,8 @@ PK_API int pk_rmsnorm_bwd(const void* d_y, const void* x, int dtype, const void*
  * (BmmExperts, qwen3_bmm_experts_patch.py:90-110).
  * Together these replace _run_bmm_experts (qwen3_bmm_experts_patch.py:11-50) and the
  * autograd graph torch builds for it (src/executors.py:257-296).
- * bf16 runs on MFMA tiles and needs H % 64 == 0 and I % 64 == 0; f32 runs on a
+ * bf16 runs on MFMA tiles when H % 128 == 0, I % 128 == 0 and every operand is 16-byte aligned,
+ * and on a shape-unrestricted FMA kernel (still HIP, same results to rounding) otherwise; f32 runs on a
  * tiled FMA kernel with no shape restriction.
  */
 

@@ -42,6 +42,7 @@ SIGNATURES = {
     "pk_rmsnorm_bwd_workspace_bytes": (_c_i64, [_c_i64, _c_i64]),
     "pk_rmsnorm_bwd": (_c_int, [_p, _p, _c_int, _p, _p, _p, _p, _p, _c_int, _c_i64, _c_i64, _p, _c_i64, _p]),
     "pk_combine_bwd": (_c_int, [_p, _p, _c_int, _p, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
+    "pk_zero_rows_from": (_c_int, [_p, _c_int, _p, _c_i64, _c_i64, _p]),
     "pk_grouped_swiglu_fwd": (_c_int, [_p, _p, _c_i64, _p, _p, _p, _p, _p, _p, _p, _p,
                                        _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
     "pk_grouped_swiglu_dgrad": (_c_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p,

@@ -1,54 +1,85 @@
 """`piper.annotate`: tag a region of model code with a schedule name (src/piper.py:51-80).
 
-Same contract as the reference: a non-empty string name, an integer index assigned per name in
-the order scopes are entered, a process-wide uid, and a stack so nested scopes ("PP" around
-"EP") are visible together.  The reference stores the stack in FX node metadata for its graph
-splitter; here the stack is what the executor reads to decide which region a call belongs to.
+Contract kept from the reference: the tag name is a non-empty string (anything else is a
+``ValueError``); every scope gets a record ``{"name", "index", "uid"}`` where ``index`` counts
+the scopes opened under that name so far and ``uid`` counts all scopes of the process; scopes
+nest ("PP" around "EP") and the active ones are visible together.  The reference writes the
+records into FX node metadata for its graph splitter; here they are what the executor reads to
+decide which region a call belongs to.
 """
 from __future__ import annotations
 
-from contextlib import contextmanager
+import itertools
+from collections import Counter
 from typing import Iterator
-
-_ANNOTATION_STACK: list[dict] = []
-_ANNOTATION_COUNTS: dict[str, int] = {}
-_ANNOTATION_UID = 0
 
 PP_TAG = "PP"
 EP_TAG = "EP"
 
 
+class _Scope:
+    """One `with annotate(name):` block.  Entering registers the record, leaving removes it."""
+
+    __slots__ = ("_registry", "_name", "record")
+
+    def __init__(self, registry: "_Registry", name: str):
+        self._registry = registry
+        self._name = name
+        self.record: dict | None = None
+
+    def __enter__(self) -> dict:
+        self.record = self._registry.open(self._name)
+        return self.record
+
+    def __exit__(self, *exc) -> bool:
+        self._registry.close(self.record)
+        return False
+
+
+class _Registry:
+    """Process-wide bookkeeping of annotation scopes."""
+
+    def __init__(self):
+        self.reset()
+
+    def reset(self) -> None:
+        self.active: list[dict] = []
+        self.per_name: Counter = Counter()
+        self.serial: Iterator[int] = itertools.count()
+
+    def open(self, name: str) -> dict:
+        record = {"name": name, "index": self.per_name[name], "uid": next(self.serial)}
+        self.per_name[name] += 1
+        self.active.append(record)
+        return record
+
+    def close(self, record: dict) -> None:
+        # scopes are context managers, so they close innermost first
+        if not self.active or self.active[-1] is not record:
+            raise RuntimeError(f"annotation scope {record!r} closed out of order")
+        self.active.pop()
+
+
+_REGISTRY = _Registry()
+
+
+def annotate(name: str) -> _Scope:
+    """Context manager that tags everything run inside it with `name`."""
+    if not (isinstance(name, str) and name):
+        raise ValueError(f"annotate() takes a non-empty string as tag name, not {name!r}")
+    return _Scope(_REGISTRY, name)
+
+
 def reset_annotation_state() -> None:
-    global _ANNOTATION_UID
-    _ANNOTATION_STACK.clear()
-    _ANNOTATION_COUNTS.clear()
-    _ANNOTATION_UID = 0
+    """Forget all scopes and restart the index / uid numbering (used between model builds)."""
+    _REGISTRY.reset()
 
 
 def current_annotations() -> tuple[dict, ...]:
     """Snapshot of the active scopes, outermost first."""
-    return tuple(dict(a) for a in _ANNOTATION_STACK)
+    return tuple(dict(r) for r in _REGISTRY.active)
 
 
 def current_tag() -> dict[str, int]:
     """{name: index} of the active scopes, e.g. {"PP": 0, "EP": 0} inside the expert region."""
-    return {a["name"]: a["index"] for a in _ANNOTATION_STACK}
-
-
-@contextmanager
-def annotate(name: str) -> Iterator[dict]:
-    if not isinstance(name, str) or not name:
-        raise ValueError(f"piper.annotate requires a non-empty string tag name, got {name!r}")
-    global _ANNOTATION_UID
-    index = _ANNOTATION_COUNTS.get(name, 0)
-    _ANNOTATION_COUNTS[name] = index + 1
-    uid = _ANNOTATION_UID
-    _ANNOTATION_UID += 1
-    annotation = {"name": name, "index": int(index), "uid": int(uid)}
-    _ANNOTATION_STACK.append(annotation)
-    try:
-        yield annotation
-    finally:
-        popped = _ANNOTATION_STACK.pop()
-        if popped is not annotation:
-            raise RuntimeError("piper.annotate stack corrupted")
+    return {r["name"]: r["index"] for r in _REGISTRY.active}

@@ -14,6 +14,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Any, Callable, Sequence
 
+import logging
+
 import torch
 
 from . import ops
@@ -28,11 +30,13 @@ class BucketState:
 
     forward_fn: Any = None
     forward_args: list = field(default_factory=list)
+    forward_input_meta: list = field(default_factory=list)
     input_idxs: list = field(default_factory=list)
     param_idxs: list = field(default_factory=list)
     param_names: list = field(default_factory=list)
     optimizer: Any = None
     trainable_param_idxs: list = field(default_factory=list)
+    activation_checkpoint_subgraph_count: int = 1
 
     flat_params: torch.Tensor | None = None          # param dtype; parameters are views of it
     flat_grads: torch.Tensor | None = None           # fp32
@@ -116,11 +120,90 @@ class StageStore:
 
 
 @dataclass
-class ParamStorage:
-    """ZeRO parameter and gradient storage of one device (src/runtime.py:202-495)."""
+class RuntimeState:
+    """The few fields of the reference's per-actor runtime record (src/runtime.py:102-200) that the
+    bucket path reads.  One GPU: rank 0 of a data-parallel group of one."""
 
-    stages: StageStore
-    grad_buffer_dtype: torch.dtype = torch.float32
+    device: Any = None
+    dp_degree: int = 1
+    dp_rank: int = 0
+    global_rank: int = 0
+    dp_group: Any = None
+
+
+class _DeferredFree:
+    """A release that has to wait for a GPU event (src/runtime.py:284-310).  The reference hands
+    `evt.synchronize(); free()` to a one-thread pool and keeps the Future; here the wait and the
+    release run when somebody asks for the result, which is what every consumer of the Future does
+    before it touches the buffer again (`wait_pending_free`, `drain_pending_frees`)."""
+
+    def __init__(self, evt, release):
+        self._evt, self._release, self._done = evt, release, False
+
+    def done(self) -> bool:
+        return self._done or self._evt is None or self._evt.query()
+
+    def result(self) -> None:
+        if self._done:
+            return
+        if self._evt is not None:
+            self._evt.synchronize()
+        self._release()
+        self._done = True
+
+
+class ParamStorage:
+    """ZeRO parameter and gradient storage of one device (src/runtime.py:202-495): same constructor
+    arguments (runtime, stages, logger), same method names and arguments.  `ParamStorage(stages)` is
+    accepted as a shorthand.  Differences that follow from running the one GPU's share with a
+    data-parallel group of one: the shard is the whole bucket, so "freeing the full parameters"
+    releases nothing and only marks the bucket stale, and gradients are packed although the
+    reference skips the pack when dp_degree <= 1 (src/runtime.py:254)."""
+
+    def __init__(self, runtime: Any = None, stages: "StageStore | None" = None, logger: Any = None,
+                 grad_buffer_dtype: torch.dtype = torch.float32):
+        if isinstance(runtime, StageStore) and stages is None:
+            runtime, stages = None, runtime
+        if stages is None:
+            raise TypeError("ParamStorage needs the StageStore of its buckets")
+        self.runtime = runtime if runtime is not None else RuntimeState()
+        self.stages = stages
+        self.logger = logger if logger is not None else logging.getLogger("piper_amd.bucket")
+        self.grad_buffer_dtype = grad_buffer_dtype
+        self.pending_param_frees: dict = {}
+        self.pending_grad_frees: dict = {}
+
+    # ---- deferred frees (src/runtime.py:231-247,284-310)
+    def wait_pending_free(self, pending: dict, ubid) -> None:
+        if ubid is None:
+            return
+        fut = pending.pop(ubid, None)
+        if fut is not None:
+            fut.result()
+
+    def drain_pending_frees(self) -> None:
+        for pending in (self.pending_param_frees, self.pending_grad_frees):
+            futures = list(pending.values())
+            pending.clear()
+            for fut in futures:
+                fut.result()
+
+    def defer_free_full_params(self, ubid, evt) -> None:
+        """Free the bucket's full parameters once `evt` has happened (the forward/backward that
+        reads them was recorded before it)."""
+        if ubid is None or ubid not in self.stages.param_sharded_ubids:
+            return
+        self.wait_pending_free(self.pending_param_frees, ubid)
+        self.pending_param_frees[ubid] = _DeferredFree(evt, lambda: self.free_full_params(ubid))
+
+    def defer_free_full_grads(self, ubid, evt) -> None:
+        if ubid is None or ubid not in self.stages.grad_sharded_ubids:
+            return
+        self.wait_pending_free(self.pending_grad_frees, ubid)
+        # the pack that recorded `evt` has already dropped the per-tensor gradients, and with a
+        # data-parallel group of one the flat buffer is also the optimizer's shard gradient: after the
+        # event nothing is left to release (a late `free_full_grads` would only wipe newer gradients)
+        self.pending_grad_frees[ubid] = _DeferredFree(evt, lambda: None)
 
     def clear_param_grads(self) -> None:
         for bucket in self.stages.buckets.values():
@@ -142,6 +225,8 @@ class ParamStorage:
         the bucket in one launch, then drop the per-tensor grads."""
         if ubid is None or ubid not in self.stages.zero_managed_ubids:
             return
+        if ubid in self.stages.grad_sharded_ubids:
+            self.wait_pending_free(self.pending_grad_frees, ubid)
         bucket = self.stages.bucket(ubid)
         specs = bucket.param_view_specs
         if not specs:
@@ -170,6 +255,7 @@ class ParamStorage:
     def alloc_full_params(self, ubid) -> None:
         """Unflatten (src/runtime.py:312-352): make every parameter a view of the flat bucket."""
         bucket = self.stages.bucket(ubid)
+        self.wait_pending_free(self.pending_param_frees, ubid)
         full = bucket.flat_params
         assert full is not None, f"alloc_full_params: missing flat_params buffer for ubid={ubid}"
         assert bucket.param_view_specs, f"alloc_full_params: missing param_view_specs for ubid={ubid}"
@@ -186,6 +272,7 @@ class ParamStorage:
 
     def alloc_full_grads(self, ubid, stream: torch.cuda.Stream | None = None) -> None:
         bucket = self.stages.bucket(ubid)
+        self.wait_pending_free(self.pending_grad_frees, ubid)
         with torch.cuda.stream(stream):
             if bucket.flat_grads is None:
                 bucket.flat_grads = torch.zeros(bucket.param_shard_info[1], dtype=self.grad_buffer_dtype,

@@ -9,7 +9,6 @@
 #include "pk_common.h"
 #include "simt_gemm.h"
 #include <atomic>
-#include <cstdlib>
 #include <initializer_list>
 #include <mutex>
 
@@ -49,7 +48,7 @@ __device__ __forceinline__ int logical_block() {
 __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off"
                :: "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr)
-               : "memory");
+               : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void wait_dma() {
@@ -431,9 +430,6 @@ struct RaggedMParams {
   float* ds_partial;     // SWIGLU_BWD_SCALED: [ldc / 64][total_rows] partial <unscaled d_h, h>
   int64_t total_rows;
   SchedSlot* sched;      // this launch's counters
-#ifdef PK_GEMM_DEBUG
-  int32_t debug;         // 1: skip MFMAs, 2: skip loads, 4: skip stores
-#endif
 };
 
 // Wave-private staging of 32 rows x COLS bf16 of the output through LDS, so that global stores
@@ -647,11 +643,6 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     }
   };
 
-#ifdef PK_GEMM_DEBUG
-  const bool dbg_loads_v = !(p.debug & 2), dbg_mma = !(p.debug & 1);
-#else
-  constexpr bool dbg_loads_v = true, dbg_mma = true;
-#endif
   // DMA of k-tile `kt` of unit `t` into ring stage `stage`: piece 0..LA-1 = A, LA..L-1 = B
   int is_k0 = 0, is_seg = 0;
   uint32_t is_a = 0, is_b = 0;
@@ -679,7 +670,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   };
   auto issue_tile = [&](const Unit& t, int kt, int stage) {
     issue_setup(kt, stage);
-    is_real = dbg_loads_v && kt < nkt;
+    is_real = kt < nkt;
 #pragma unroll
     for (int i = 0; i < L; ++i) issue_piece(t, i);
   };
@@ -727,10 +718,10 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
       }
       const int tgt = cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1;   // stage of k-tile kt-1 = kt+NS-1
       issue_setup(kt + NS - 1, tgt);
-      is_real = dbg_loads_v && kt + NS - 1 < nkt;
+      is_real = kt + NS - 1 < nkt;
       const char* st = smem + cur * STAGE;
       const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
-      if (wave_has_rows && dbg_mma) {
+      if (wave_has_rows) {
         mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN,
                                                      f0, acc, [&](int piece) { issue_piece(cur_u, piece); });
       } else {
@@ -758,11 +749,6 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     const int lrow = lane & 31, lq = 4 * (lane >> 5);
     const int64_t grow0 = (int64_t)(cur_u.row0 + wm * WTM) * p.ldc;
     const int64_t gcol0 = (int64_t)cur_u.nt * BN_OUT + wn * OUT_COLS;
-#ifdef PK_GEMM_DEBUG
-    const bool do_store = !(p.debug & 4);
-#else
-    constexpr bool do_store = true;
-#endif
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int crows = min(32, cur_u.rows - wm * WTM - 32 * i);   // valid rows of this chunk
@@ -770,7 +756,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
       if (EPI == EPI_SWIGLU) {
 #pragma unroll
         for (int which = 0; which < 3; ++which) {
-          if (crows > 0 && do_store) {
+          if (crows > 0) {
 #pragma unroll
             for (int j = 0; j < TN; j += 2)
 #pragma unroll
@@ -793,7 +779,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
           }
         }
       } else if (EPI == EPI_PLAIN) {
-        if (crows > 0 && do_store) {
+        if (crows > 0) {
 #pragma unroll
           for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -840,7 +826,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
         // the loads above must have returned first: a load behind the prefetch waits for all of it
         __builtin_amdgcn_sched_barrier(0);
         if (i == TM - 1) prefetch_next();
-        if (crows > 0 && do_store) {
+        if (crows > 0) {
           if (SCALED) {
             // lanes l and l+32 hold the two column halves of row l % 32
             ds += __shfl_xor(ds, 32);
@@ -887,9 +873,6 @@ struct WgradParams {
   int32_t accumulate;
   int32_t tiles_per_expert;  // (M/BM)*(N/BN), identical for the three problems
   int32_t nprob;
-#ifdef PK_GEMM_DEBUG
-  int32_t debug;
-#endif
 };
 
 template <int BM, int BN, int BK, int WMW, int WNW, int NS>
@@ -1062,24 +1045,15 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
     for (int kt = 0; kt < nkt; ++kt) {
       if (kt + NS - 2 < nkt) wait_dma<(NS - 2) * (LA + LB)>(); else wait_dma<0>();
       block_barrier();
-#ifdef PK_GEMM_DEBUG
-      if (!(p.debug & 2))
-#endif
       if (kt + NS - 1 < nkt) issue(nxt);
       if (kt + NS < nkt) fetch_rows(kt + NS);
       const char* st = smem + cur * STAGE;
-#ifdef PK_GEMM_DEBUG
-      if (!(p.debug & 1))
-#endif
       mma_tile<BK, TM, TN, false, false, BM, BN, (TM * TN >= 16)>(st, st + A_BYTES, wm * WTM, wn * WTN, acc);
       cur = cur + 1 == NS ? 0 : cur + 1;
       nxt = nxt + 1 == NS ? 0 : nxt + 1;
     }
   }
 
-#ifdef PK_GEMM_DEBUG
-  if (p.debug & 4) { if (acc[0][0][0] != 12345.678f) return; }
-#endif
   block_barrier();
   bf16_t* C = q.C + (int64_t)e * q.M * q.N + ((int64_t)mt * BM + wm * WTM) * q.N + (int64_t)nt * BN + wn * WTN;
   char* sbuf = smem + wave * (WTM * St::LD);
@@ -1135,9 +1109,6 @@ inline SchedSlot* sched_slot_for_launch() {
 
 template <int BM, int BN, int BK, int WMW, int WNW, int NS, bool B_KC, int EPI>
 int launch_ragged_m(RaggedMParams p, int64_t A_rows, int kernel_id, hipStream_t s) {
-#ifdef PK_GEMM_DEBUG
-  { const char* d = getenv("PK_GEMM_DEBUG_MODE"); p.debug = d ? atoi(d) : 0; }
-#endif
   const int64_t max_units = (pk_ceil_div(A_rows, BM) + p.E) * p.n_tiles;
   if (max_units > 0x7ffffff0ll || p.ldb * (int64_t)(BN > BK ? BN : BK) > 0x7fffffffll) return PK_ERR_SHAPE;
   if ((int64_t)p.Kseg * p.nseg < 2 * BK) return PK_ERR_SHAPE;   // the k-loop publishes the next unit in its second step
@@ -1246,30 +1217,27 @@ int simt_ragged_k(const void* A, int64_t lda, const int32_t* a_map, const void* 
   return pk_simt::launch<T, T, T>(p, s);
 }
 
-// Tile configurations: BM, BN, waves along M, waves along N, LDS stages.  Measured on MI355X
-// with random data and multinomial / Zipf row counts over {128,256}x{128,256} tiles, 4/8/16
-// waves and 2/3 stages: 128x256 with 8 waves (64x64 wave tiles, 3-stage 144 KB ring) is fastest
-// for the ragged-M kernels, 256x256 with 8 waves (128x64 wave tiles) for the weight gradient.
-// (BM, BN, BK, waves M, waves N, stages, workgroups per CU)
-#ifndef PK_RM_CFG
+// Tile configurations (BM, BN, BK, waves along M, waves along N, LDS ring stages), chosen by
+// measurement on MI355X with random data and multinomial / Zipf row counts.
+// Ragged-M kernels: 256x256x32 block tiles, 8 waves (128x64 wave tiles), 4-stage 128 KB ring.
 #define PK_RM_CFG 256, 256, 32, 2, 4, 4
 #define PK_RM_BN 256
-/* same width, 128 rows: for launches with few 256-row units per workgroup */
+// Same width with 128 rows and a 5-stage ring: for launches that would give a workgroup fewer than
+// PK_RM_LOWM_UNITS of the 256-row units, and for the scaled SwiGLU backward.
 #define PK_RM_LOWM 128, 256, 32, 2, 4, 5
 #define PK_RM_LOWM_UNITS 3
-#endif
-#ifndef PK_WG_BIG
-#define PK_WG_BIG 256, 256, 64, 2, 4, 2     /* 8 waves, 128x64 wave tiles, 128 KB ring */
+// Output widths that are a multiple of 128 but not of 256.
+#define PK_RM_ALT 128, 128, 64, 2, 2, 4
+// Weight gradient: 256x256x64 in a 2-stage ring; with fewer than PK_WG_SHORTK_ROWS rows per expert on
+// average 32-deep tiles in a 4-stage ring with the loads spread between the MFMAs (measured
+// against the 64-deep ring: -1.8 % at 256 rows per expert, +7 % at 1,024).
+#define PK_WG_BIG 256, 256, 64, 2, 4, 2
 #define PK_WG_BIG_THREADS 512
-#endif
-/* short reductions (few rows per expert): 32-deep tiles in a 4-stage ring, loads spread between the
-   MFMAs; measured against the 64-deep 2-stage ring: -1.8 % at 256 rows per expert, +7 % at 1,024 */
 #define PK_WG_BIG_SHORTK 256, 256, 32, 2, 4, 4
 #define PK_WG_SHORTK_ROWS 512
 #define PK_WG_SMALL 128, 128, 64, 2, 2, 4
 #define PK_WG_SMALL_THREADS 256
 
-#define PK_RM_ALT 128, 128, 64, 2, 2, 4      /* output widths that are a multiple of 128 but not of 256 */
 bool mfma_shape_ok(int64_t H, int64_t I) { return H % 128 == 0 && I % 128 == 0; }
 
 // Pick the tile width by the output width N of the GEMM (for the gate/up kernel a tile holds
@@ -1542,9 +1510,6 @@ static int wgrad_impl(const void* d_y, int dy_gathered, const void* h, const voi
   if (n == 0) return PK_OK;
   p.starts = starts; p.order = expert_order; p.E = (int32_t)E; p.map_div = mf::make_fastdiv(row_map_div);
   p.accumulate = accumulate ? 1 : 0;
-#ifdef PK_GEMM_DEBUG
-  { const char* d = getenv("PK_GEMM_DEBUG_MODE"); p.debug = d ? atoi(d) : 0; }
-#endif
   const bool big = (H % 256 == 0) && (I % 256 == 0);
   const int tile = big ? 256 : 128;
   p.tiles_per_expert = (int32_t)((H / tile) * (I / tile));

@@ -301,9 +301,36 @@ int rmsnorm_bwd_launch(const void* d_y, const void* x, const void* weight, const
   return PK_OK;
 }
 
+// buf[r, :] = 0 for r in [*first_row, rows): the rows of an expert-sorted buffer that no expert
+// owns.  The first row is read on the device, so the grid is fixed and the blocks stride the rows.
+__global__ __launch_bounds__(kRowThreads) void zero_rows_from_kernel(char* __restrict__ buf, const int32_t* __restrict__ first_row,
+                                                                     int64_t rows, int64_t row_bytes) {
+  for (int64_t r = (int64_t)*first_row + blockIdx.x; r < rows; r += gridDim.x) {
+    char* row = buf + r * row_bytes;
+    if ((row_bytes & 15) == 0 && (((uintptr_t)buf) & 15) == 0) {
+      const u32x4_t z = {0u, 0u, 0u, 0u};
+      for (int64_t v = threadIdx.x; v < row_bytes / 16; v += kRowThreads) reinterpret_cast<u32x4_t*>(row)[v] = z;
+    } else {
+      for (int64_t v = threadIdx.x; v < row_bytes; v += kRowThreads) row[v] = 0;
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" {
+
+int pk_zero_rows_from(void* buf, int dtype, const int32_t* first_row, int64_t rows, int64_t width, pk_stream_t stream) {
+  if (rows < 0 || width <= 0 || !pk_dtype_ok(dtype)) return PK_ERR_ARG;
+  if (rows == 0) return PK_OK;
+  if (!buf || !first_row) return PK_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned grid = (unsigned)(rows < 512 ? rows : 512);
+  PK_LAUNCH_NOCHECK(pk_timing::K_MISC, s, zero_rows_from_kernel, dim3(grid), dim3(kRowThreads), 0, s, (char*)buf, first_row,
+                    rows, width * (int64_t)pk_dtype_size(dtype));
+  PK_RETURN_IF_LAUNCH_FAILED();
+  return PK_OK;
+}
 
 int pk_permute_fwd(const void* x, int dtype, const int32_t* perm, void* routed, int64_t A,
                    int64_t H, int64_t K, pk_stream_t stream) {

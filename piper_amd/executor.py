@@ -21,68 +21,83 @@ from .planner import plan_zero_lifetimes
 from .tasks import COMM_TASKS, TaskType
 
 
+def _as_list(value) -> list:
+    if isinstance(value, (list, tuple)):
+        return list(value)
+    return [value]
+
+
+def _wants_grad(t) -> bool:
+    return isinstance(t, torch.Tensor) and t.requires_grad
+
+
+def _cut(t):
+    """A leaf that shares t's storage: autograd stops here, and the leaf collects the gradient that
+    the consumer's backward produces for t."""
+    return t.detach().requires_grad_(True) if _wants_grad(t) else t
+
+
 @dataclass
 class ComputeExecutor:
-    """Bucket forward/backward execution (src/executors.py:169-296)."""
+    """Forward / backward of one bucket with the call contract of the reference's executor
+    (src/executors.py:169-296): same arguments, same keys in the returned dictionaries."""
 
     stages: StageStore
 
     def forward(self, ubid: Any, input_tensors: Any, compute_stream: torch.cuda.Stream | None = None) -> dict:
+        """Run the bucket's forward function on `compute_stream`.
+
+        Each input that takes part in autograd enters as a fresh leaf, and each such output is handed
+        on as a fresh leaf as well ("detached_outs"), so every bucket owns a closed autograd graph
+        whose ends exchange gradients through `.grad`."""
         bucket = self.stages.bucket(ubid)
-        fwd_fn, fwd_args, input_idxs = bucket.forward_fn, bucket.forward_args, bucket.input_idxs
-        if not isinstance(input_tensors, (list, tuple)):
-            input_tensors = [input_tensors]
-        for i, tensor in zip(input_idxs, input_tensors):
-            if isinstance(tensor, (list, tuple)):
-                tensor = tensor[0]
-            if tensor.requires_grad:
-                tensor = tensor.detach().requires_grad_(True)
-            fwd_args[i] = tensor
-        fwd_inputs = [fwd_args[i] for i in input_idxs]
-        inp_with_grad = [t for t in fwd_inputs if t is not None and t.requires_grad]
-        with torch.cuda.stream(compute_stream):
-            output = fwd_fn(fwd_args)
-        for i in input_idxs:
-            fwd_args[i] = None
-        out_list = list(output) if isinstance(output, tuple) else [output]
-        possibly_detached = [
-            t.detach().requires_grad_(True) if isinstance(t, torch.Tensor) and t.requires_grad else t
-            for t in out_list
-        ]
-        out_with_grad = [t for t in out_list if isinstance(t, torch.Tensor) and t.requires_grad]
+        args, slots = bucket.forward_args, list(bucket.input_idxs)
+        leaves = []
+        for value in _as_list(input_tensors)[:len(slots)]:
+            # a producer may hand over its whole output list; the boundary tensor is its head
+            leaves.append(_cut(_as_list(value)[0]))
+        for slot, leaf in zip(slots, leaves):
+            args[slot] = leaf
+        fwd_inputs = [args[slot] for slot in slots]
+        try:
+            with torch.cuda.stream(compute_stream):
+                result = bucket.forward_fn(args)
+        finally:
+            for slot in slots:            # activations must not stay alive inside the argument list
+                args[slot] = None
+        outs = _as_list(result)
         return {
-            "pre_detach_outs": out_list,
-            "detached_outs": possibly_detached,
-            "out_with_grad": out_with_grad,
-            "send_output": output,
-            "inp_with_grad": inp_with_grad,
+            "pre_detach_outs": outs,
+            "detached_outs": [_cut(t) for t in outs],
+            "out_with_grad": [t for t in outs if _wants_grad(t)],
+            "send_output": result,
+            "inp_with_grad": [t for t in fwd_inputs if _wants_grad(t)],
             "fwd_inputs": fwd_inputs,
         }
 
     def backward(self, ubid: Any, mb_idx: int, outputs_or_loss: list, upstream_grads: Any,
                  pre_detach_outs: Any, detached_outs: Any, inp_with_grad: Any, out_with_grad: Any,
                  compute_stream: torch.cuda.Stream | None = None) -> dict | None:
+        """Backward of one bucket.  Without `pre_detach_outs` the roots are `outputs_or_loss` (a loss,
+        or outputs with explicit `upstream_grads`); with them, the roots are the bucket's own outputs
+        and their gradients are whatever the consumer left in `.grad` of the detached copies.
+        Returns {"send_output": input gradients} when the bucket has inputs that received one."""
         if pre_detach_outs is None:
-            with torch.cuda.stream(compute_stream):
-                if upstream_grads is not None:
-                    torch.autograd.backward(outputs_or_loss, upstream_grads)
-                else:
-                    outputs_or_loss[0].backward()
+            roots = list(outputs_or_loss) if upstream_grads is not None else [outputs_or_loss[0]]
+            grads = upstream_grads
         else:
-            bwd_pairs = [
-                (p, d.grad) for p, d in zip(pre_detach_outs, detached_outs)
-                if isinstance(d, torch.Tensor) and d.requires_grad and d.grad is not None
-            ]
-            assert bwd_pairs, (
-                f"BWD ubid={ubid} mb={mb_idx}: detached boundary has no tensors with a materialized grad"
-            )
-            with torch.cuda.stream(compute_stream):
-                torch.autograd.backward([p for p, _ in bwd_pairs], [g for _, g in bwd_pairs])
-        if inp_with_grad:
-            output_grads = [t.grad for t in inp_with_grad if t.grad is not None]
-            if output_grads:
-                return {"send_output": output_grads}
-        return None
+            roots, grads = [], []
+            for produced, handed_on in zip(pre_detach_outs, detached_outs):
+                if _wants_grad(handed_on) and handed_on.grad is not None:
+                    roots.append(produced)
+                    grads.append(handed_on.grad)
+            if not roots:
+                raise AssertionError(f"backward of bucket {ubid!r}, microbatch {mb_idx}: no output of the "
+                                     "bucket received a gradient from its consumer")
+        with torch.cuda.stream(compute_stream):
+            torch.autograd.backward(roots, grads)
+        received = [t.grad for t in (inp_with_grad or ()) if t.grad is not None]
+        return {"send_output": received} if received else None
 
 
 @dataclass
@@ -126,8 +141,15 @@ class StageExecutor:
         """Run one training iteration.  ``microbatches[mb]`` feeds the first bucket's forward; each
         bucket's detached output feeds the next bucket; the last bucket's output goes to ``loss_fn``
         (or is summed when there is no loss_fn)."""
-        cs = self.compute_stream or torch.cuda.current_stream()
+        caller = torch.cuda.current_stream()
+        cs = self.compute_stream or caller
         ps = self.pack_stream or cs
+        # the microbatches (and whatever else the caller queued) were produced on the caller's stream
+        if cs != caller:
+            cs.wait_stream(caller)
+        if ps != caller and ps is not cs:
+            ps.wait_stream(caller)
+        self.params.drain_pending_frees()        # src/executors.py:584
         self._fwd.clear()
         self._inp_grads.clear()
         self._wgrad_queues.clear()
@@ -154,8 +176,8 @@ class StageExecutor:
                 if task.ubid in self.stages.param_sharded_ubids and life.gather_params_before:
                     self.params.all_gather_full_params(task.ubid, cs)
                 self._fwd[(task.ubid, task.mb)] = self.compute.forward(task.ubid, inp, cs)
-                if task.ubid in self.stages.param_sharded_ubids and life.free_params_after:
-                    self.params.free_full_params(task.ubid)
+                if life.free_params_after:
+                    self._free_params_after(task.ubid, cs)
             elif tt in (TaskType.BWD, TaskType.FWD_BWD, TaskType.BWD_I):
                 # BWD_I is the same walk with the weight gradients of the HIP operators queued
                 # instead of computed (src/executors.py:353-411); BWD_W runs the queue (:413-476)
@@ -195,21 +217,30 @@ class StageExecutor:
                     self._wgrad_queues[(task.ubid, task.mb)] = queue
                 if life.reduce_grads_after:
                     self._pack_after_backward(task.ubid, cs, ps, pack_events)
-                if task.ubid in self.stages.param_sharded_ubids and life.free_params_after:
-                    self.params.free_full_params(task.ubid)
+                if life.free_params_after:
+                    self._free_params_after(task.ubid, cs)
             elif tt is TaskType.BWD_W:
                 queue = self._wgrad_queues.pop((task.ubid, task.mb))
                 with torch.cuda.stream(cs):
                     queue.run()
                 if life.reduce_grads_after:
                     self._pack_after_backward(task.ubid, cs, ps, pack_events)
-                if task.ubid in self.stages.param_sharded_ubids and life.free_params_after:
-                    self.params.free_full_params(task.ubid)
+                if life.free_params_after:
+                    self._free_params_after(task.ubid, cs)
             elif tt is TaskType.UPD:
                 self._update(cs, pack_events)
             else:
                 raise NotImplementedError(f"task {tt} is not a per-device task of this executor")
         return {"losses": losses}
+
+    def _free_params_after(self, ubid, cs) -> None:
+        """Release the bucket's full parameters once the compute task just queued on `cs` has run
+        (src/executors.py:769-774,876)."""
+        if ubid not in self.stages.param_sharded_ubids:
+            return
+        evt = torch.cuda.Event()
+        evt.record(cs)
+        self.params.defer_free_full_params(ubid, evt)
 
     def _pack_after_backward(self, ubid, cs, ps, pack_events: dict) -> None:
         """Gradient pack on the second stream, ordered after the backward that produced the grads."""
@@ -217,14 +248,17 @@ class StageExecutor:
             evt = torch.cuda.Event()
             evt.record(cs)
             ps.wait_event(evt)
-        self.params.accumulate_zero_param_grads_to_flat(ubid, ps if ps is not cs else None)
+        self.params.accumulate_zero_param_grads_to_flat(ubid, ps)
         if ps is not cs:
             done = torch.cuda.Event()
             done.record(ps)
             pack_events[ubid] = done
+            if ubid in self.stages.grad_sharded_ubids:
+                self.params.defer_free_full_grads(ubid, done)     # src/executors.py:719
 
     def _update(self, stream, pack_events: dict):
         """src/executors.py:1005-1034."""
+        self.params.drain_pending_frees()
         if self.params.has_zero_shard_optimizers():
             self.params.step_zero_shard_optimizers(stream, pack_events)
         for bucket in self.stages.buckets.values():

@@ -44,21 +44,42 @@ class _RouterFn(torch.autograd.Function):
         return d_x, d_w, d_b, None, None, None
 
 
+def _sorted_tables(top_idx: torch.Tensor, num_experts: int):
+    """(counts, starts, perm, inv_perm) of the counting sort of `top_idx`, computed once per routing
+    result: the tables ride on the index tensor, and the inverse permutation rides on `perm`, so the
+    piecewise operators that follow (reorder, permute backward, combine) launch no second sort."""
+    cached = getattr(top_idx, "_pk_sorted", None)
+    if cached is None or cached[0].numel() != num_experts:
+        cached = ops.sort_by_expert(top_idx, num_experts)
+        cached[2]._pk_inverse = cached[3]
+        top_idx._pk_sorted = cached
+    return cached
+
+
+def _inverse_of(perm: torch.Tensor) -> torch.Tensor:
+    """inv_perm for a permutation produced by `reorder` (cached there); any other permutation is
+    inverted once and remembered on the tensor."""
+    inv = getattr(perm, "_pk_inverse", None)
+    if inv is None:
+        inv = torch.empty_like(perm)
+        inv[perm.long()] = torch.arange(perm.numel(), dtype=perm.dtype, device=perm.device)
+        perm._pk_inverse = inv
+    return inv
+
+
 def router(x, w_gate, gate_bias=None, *, top_k: int, route_norm: bool, route_scale: float = 1.0):
     """(top_scores [T,K] f32, selected_experts_indices [T,K] i32, num_tokens_per_expert [E] i32).
-    The call `self.router(x, self.expert_bias)` of qwen3.py:237-241."""
+    The call `self.router(x, self.expert_bias)` of qwen3.py:237-241.  The histogram is the one the
+    counting sort produces (no host sync, no second pass over the indices)."""
     top_scores, top_idx = _RouterFn.apply(x, w_gate, gate_bias, top_k, route_norm, route_scale)
-    # histogram without a host sync (torch.bincount reads the maximum back to size its output)
-    flat = top_idx.reshape(-1)
-    counts = torch.zeros(w_gate.shape[0], dtype=torch.int32, device=flat.device)
-    counts.index_add_(0, flat, torch.ones_like(flat))
+    counts = _sorted_tables(top_idx, w_gate.shape[0])[0]
     return top_scores, top_idx, counts
 
 
 def reorder(top_scores: torch.Tensor, top_idx: torch.Tensor, num_experts: int):
     """The reorderer of qwen3.py:243-247.  Returns (top_scores_experts_sorted [A],
     token_indices_experts_sorted [A] i32, num_tokens_per_expert [E] i32)."""
-    counts, _starts, perm, _inv = ops.sort_by_expert(top_idx, num_experts)
+    counts, _starts, perm, _inv = _sorted_tables(top_idx, num_experts)
     scores_sorted = top_scores.reshape(-1)[perm.long()]
     return scores_sorted, perm, counts
 
@@ -67,15 +88,12 @@ class _PermuteFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, perm, top_k):
         ctx.top_k = top_k
-        ctx.save_for_backward(perm)
+        ctx.inv_perm = _inverse_of(perm)
         return ops.permute_fwd(x, perm, top_k)
 
     @staticmethod
     def backward(ctx, d_routed):
-        (perm,) = ctx.saved_tensors
-        inv = torch.empty_like(perm)
-        inv[perm.long()] = torch.arange(perm.numel(), dtype=perm.dtype, device=perm.device)
-        return ops.permute_bwd(d_routed, inv, ctx.top_k), None, None
+        return ops.permute_bwd(d_routed, ctx.inv_perm, ctx.top_k), None, None
 
 
 def permute(x: torch.Tensor, token_indices_experts_sorted: torch.Tensor, top_k: int) -> torch.Tensor:
@@ -88,6 +106,9 @@ class _BmmExpertsFn(torch.autograd.Function):
     def forward(ctx, w1, w2, w3, x, num_tokens_per_expert):
         starts = ops.counts_to_starts(num_tokens_per_expert)
         y, g, u, h = ops.grouped_swiglu_fwd(x, w1, w2, w3, starts)
+        # rows past sum(num_tokens_per_expert) belong to no expert: zeros, as in the reference
+        # (qwen3_bmm_experts_patch.py:43); the kernels only write rows below starts[E]
+        ops.zero_rows_from(y, starts[-1:])
         ctx.save_for_backward(w1, w2, w3, x, starts, g, u, h)
         ctx.params = (w1, w2, w3)
         return y
@@ -96,6 +117,7 @@ class _BmmExpertsFn(torch.autograd.Function):
     def backward(ctx, d_y):
         w1, w2, w3, x, starts, g, u, h = ctx.saved_tensors
         d_x, d_g, d_u = ops.grouped_swiglu_dgrad(d_y, w1, w2, w3, g, u, starts)
+        ops.zero_rows_from(d_x, starts[-1:])
         d_w1 = d_w2 = d_w3 = None
         if all(ctx.needs_input_grad[:3]) and _can_defer(*ctx.params):
             _queue_expert_wgrad(ctx.params, d_y, h, d_g, d_u, x, starts, None, 1, None)
@@ -152,7 +174,9 @@ def _bmm_experts_forward_only(w1, w2, w3, x, num_tokens_per_expert):
     if _traced_without_data(w1, w2, w3, x, num_tokens_per_expert):
         return torch.empty_like(x)
     starts = ops.counts_to_starts(num_tokens_per_expert)
-    return ops.grouped_swiglu_fwd(x, w1, w2, w3, starts)[0]
+    y = ops.grouped_swiglu_fwd(x, w1, w2, w3, starts)[0]
+    ops.zero_rows_from(y, starts[-1:])
+    return y
 
 
 def _bmm_experts_meta(w1, w2, w3, x, num_tokens_per_expert):
@@ -194,10 +218,8 @@ def bmm_experts(w1, w2, w3, x, num_tokens_per_expert):
 class _CombineFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, y_sorted, perm, top_scores):
-        inv = torch.empty_like(perm)
-        inv[perm.long()] = torch.arange(perm.numel(), dtype=perm.dtype, device=perm.device)
         ctx.save_for_backward(y_sorted, perm, top_scores)
-        return ops.combine_fwd(y_sorted, inv, top_scores)
+        return ops.combine_fwd(y_sorted, _inverse_of(perm), top_scores)
 
     @staticmethod
     def backward(ctx, d_out):
@@ -330,18 +352,25 @@ class _ExpertRegionFn(torch.autograd.Function):
             d_x = ops.permute_bwd(d_xs, inv_perm, top_k, addend_f32=d_x32) if need[0] else None
 
             def run_router():
-                acc = p_gate.grad is not None
-                gw = p_gate.grad if acc else torch.empty_like(p_gate)
-                gb = None
-                if p_bias is not None:
-                    if p_bias.grad is not None:
-                        gb = p_bias.grad if acc else p_bias.grad.clone()
-                    else:
-                        gb = torch.zeros_like(p_bias, dtype=torch.float32) if acc else torch.empty_like(p_bias, dtype=torch.float32)
-                ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=False, d_w_gate=gw, d_gate_bias=gb, accumulate=acc)
-                p_gate.grad = gw
-                if p_bias is not None:
-                    p_bias.grad = gb
+                # the gate weight and the bias may be at different points of their accumulation
+                # (one of them cleared, the other not); the kernel has one flag for both
+                have_w = p_gate.grad is not None
+                have_b = p_bias is not None and p_bias.grad is not None
+                if p_bias is None or have_w == have_b:
+                    gw = p_gate.grad if have_w else torch.empty_like(p_gate)
+                    gb = None
+                    if p_bias is not None:
+                        gb = p_bias.grad if have_b else torch.empty_like(p_bias, dtype=torch.float32)
+                    ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=False, d_w_gate=gw, d_gate_bias=gb, accumulate=have_w)
+                    p_gate.grad = gw
+                    if p_bias is not None:
+                        p_bias.grad = gb
+                    return
+                gw = torch.empty_like(p_gate)
+                gb = torch.empty_like(p_bias, dtype=torch.float32)
+                ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=False, d_w_gate=gw, d_gate_bias=gb, accumulate=False)
+                p_gate.grad = p_gate.grad.add_(gw) if have_w else gw
+                p_bias.grad = p_bias.grad.add_(gb) if have_b else gb
 
             _WGRAD_QUEUE.push(run_router)
             return d_x, None, None, None, None, None, None, None, None, (d_out if need[9] else None)

@@ -203,6 +203,15 @@ def combine_bwd(d_out: torch.Tensor, y_sorted: torch.Tensor, perm: torch.Tensor,
     return d_y, d_scores
 
 
+def zero_rows_from(buf: torch.Tensor, first_row: torch.Tensor) -> None:
+    """buf[r] = 0 for r >= first_row[0]; first_row is a one-element int32 device tensor (no host sync)."""
+    require_gpu(buf)
+    _check(buf.dim() == 2 and buf.is_contiguous(), "zero_rows_from: contiguous [rows, width] buffer")
+    _check(first_row.dtype == torch.int32 and first_row.numel() >= 1, "zero_rows_from: int32 device scalar")
+    call("pk_zero_rows_from", ptr(buf), dtype_code(buf.dtype), ptr(first_row), buf.shape[0], buf.shape[1],
+         current_stream(buf.device))
+
+
 # ------------------------------------------------------------------------- grouped SwiGLU experts
 def _expert_dims(w1, w2, w3):
     _check(w1.dim() == 3 and w2.dim() == 3 and w3.dim() == 3, "expert weights must be [E,I,H], [E,H,I], [E,I,H]")

@@ -25,6 +25,29 @@ class PlannedBucket:
     last_use: int             # index of the last one
     members: list[int]        # parameter indices, in the order the buckets were merged
 
+    @classmethod
+    def of(cls, members: Sequence[int], use_ranges: Sequence[tuple[int, int]]) -> "PlannedBucket":
+        return cls(min(use_ranges[i][0] for i in members), max(use_ranges[i][1] for i in members), list(members))
+
+    def absorb(self, other: "PlannedBucket") -> None:
+        """Join a bucket that starts no earlier than this one."""
+        self.last_use = max(self.last_use, other.last_use)
+        self.members += other.members
+
+
+def _fill_by_bytes(sizes: Sequence[int], limit: int) -> list[list[int]]:
+    """Cut the parameter sequence into runs: a run is closed in front of the parameter that would
+    take it over `limit` bytes, unless the run holds no bytes yet (src/bucket.py:76-86)."""
+    runs: list[list[int]] = [[]]
+    used = 0
+    for i, nbytes in enumerate(sizes):
+        if used > 0 and used + nbytes > limit:
+            runs.append([])
+            used = 0
+        runs[-1].append(i)
+        used += nbytes
+    return runs
+
 
 def plan_param_buckets(sizes: Sequence[int], use_ranges: Sequence[tuple[int, int]] | None = None,
                        bucket_size_bytes: int = DEFAULT_BUCKET_BYTES,
@@ -37,11 +60,12 @@ def plan_param_buckets(sizes: Sequence[int], use_ranges: Sequence[tuple[int, int
                    True when the stage may not be cut there (the reference forbids cuts that an alias
                    of a parameter or a bfloat16_* cast crosses, src/bucket.py:250-269)
 
-    Stages, as in the reference: (1) greedy by cumulative bytes — a parameter opens a new bucket when
-    adding it would exceed the threshold and the bucket is not empty (:76-86); (2) a parameter whose
-    first and last use fall into different initial buckets becomes a bucket of its own (:88-108);
-    (3) buckets are sorted by first use and merged while their use ranges overlap (:110-128);
-    (4) neighbouring buckets are merged while the cut between them is forbidden (:250-269).
+    The result equals the reference's assignment (src/bucket.py:76-128,250-269):
+      * runs of consecutive parameters filled up to the byte threshold;
+      * a parameter that is first read inside one run's span of compute nodes and last read inside
+        another's leaves its run and stands alone;
+      * what remains is ordered by first use, and neighbours whose spans overlap are joined;
+      * neighbours are joined as well wherever the cut between them is forbidden.
     """
     n = len(sizes)
     if use_ranges is None:
@@ -50,70 +74,41 @@ def plan_param_buckets(sizes: Sequence[int], use_ranges: Sequence[tuple[int, int
         raise ValueError("plan_param_buckets: one use range per parameter")
     if bucket_size_bytes <= 0:
         raise ValueError("plan_param_buckets: bucket_size_bytes must be positive")
+    if any(first > last for first, last in use_ranges):
+        raise ValueError("plan_param_buckets: use range with first > last")
     if n == 0:
         return []
-    for lo, hi in use_ranges:
-        if lo > hi:
-            raise ValueError("plan_param_buckets: use range with first > last")
 
-    # (1) greedy
-    bucket_id = [0] * n
-    cur_b, cur_sz = 0, 0
-    for i, sz in enumerate(sizes):
-        if cur_sz + sz > bucket_size_bytes and cur_sz > 0:
-            cur_b += 1
-            cur_sz = 0
-        bucket_id[i] = cur_b
-        cur_sz += sz
-    n_init = cur_b + 1
+    runs = _fill_by_bytes(sizes, bucket_size_bytes)
+    spans = [PlannedBucket.of(run, use_ranges) for run in runs]
 
-    # (2) singleton promotion, against the ranges of the INITIAL buckets
-    init_ranges = []
-    for b in range(n_init):
-        ms = [i for i in range(n) if bucket_id[i] == b]
-        init_ranges.append((min(use_ranges[i][0] for i in ms), max(use_ranges[i][1] for i in ms)))
+    def home_run(node: int) -> int:
+        """The first run whose span covers compute node `node` (run 0 when none does)."""
+        return next((r for r, sp in enumerate(spans) if sp.first_use <= node <= sp.last_use), 0)
 
-    def bucket_at(idx: int) -> int:
-        for b, (lo, hi) in enumerate(init_ranges):
-            if lo <= idx <= hi:
-                return b
-        return 0
+    straddlers = [i for i, (first, last) in enumerate(use_ranges) if home_run(first) != home_run(last)]
+    loners = set(straddlers)
+    groups = [[i for i in run if i not in loners] for run in runs] + [[i] for i in straddlers]
+    pending = sorted((PlannedBucket.of(g, use_ranges) for g in groups if g), key=lambda b: b.first_use)
 
-    next_id = n_init
-    for i in range(n):
-        lo, hi = use_ranges[i]
-        if bucket_at(lo) != bucket_at(hi):
-            bucket_id[i] = next_id
-            next_id += 1
-
-    # (3) sort by first use (stable), merge overlapping ranges
-    groups: dict[int, list[int]] = {}
-    for i in range(n):
-        groups.setdefault(bucket_id[i], []).append(i)
-    blist = [PlannedBucket(min(use_ranges[i][0] for i in ms), max(use_ranges[i][1] for i in ms), list(ms))
-             for ms in groups.values()]
-    blist.sort(key=lambda b: b.first_use)
-    merged: list[PlannedBucket] = []
-    for b in blist:
-        if merged and b.first_use <= merged[-1].last_use:
-            prev = merged[-1]
-            merged[-1] = PlannedBucket(prev.first_use, max(prev.last_use, b.last_use), prev.members + b.members)
+    joined: list[PlannedBucket] = []
+    for bucket in pending:      # sorted() is stable: runs keep their order, loners follow them
+        if joined and bucket.first_use <= joined[-1].last_use:
+            joined[-1].absorb(bucket)
         else:
-            merged.append(b)
+            joined.append(bucket)
+    if cut_forbidden is None:
+        return joined
 
-    # (4) forbidden cuts
-    if cut_forbidden is not None:
-        changed = True
-        while changed and len(merged) > 1:
-            changed = False
-            for s in range(1, len(merged)):
-                if cut_forbidden(merged[s - 1].last_use, merged[s].first_use):
-                    prev, cur = merged[s - 1], merged[s]
-                    merged[s - 1] = PlannedBucket(prev.first_use, cur.last_use, prev.members + cur.members)
-                    del merged[s]
-                    changed = True
-                    break
-    return merged
+    # A join never changes the first use of the left neighbour and takes over the last use of the
+    # right one, so one sweep from the left sees every cut exactly as a repeated search would.
+    final: list[PlannedBucket] = []
+    for bucket in joined:
+        if final and cut_forbidden(final[-1].last_use, bucket.first_use):
+            final[-1].absorb(bucket)
+        else:
+            final.append(bucket)
+    return final
 
 
 def bucket_layers(layer_param_bytes: Sequence[Sequence[int]],
