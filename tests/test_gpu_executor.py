@@ -87,7 +87,7 @@ def _make_executor(layers, xs, dev, dtype, two_streams):
     compute_ubids = [0, 1]
     # gate buckets have no forward of their own: they are packed right after their stage's backward
     ex = StageExecutor(store, compute_stream=torch.cuda.Stream() if two_streams else None,
-                       pack_stream=torch.cuda.Stream() if two_streams else None)
+                       pack_stream=torch.cuda.Stream() if two_streams is True else None)
     # the executor walks store.buckets in order for FWD chaining: restrict chaining to compute buckets
     ex_ubids = compute_ubids
 
@@ -151,6 +151,56 @@ def test_two_bucket_1f1b_iteration(dev, dtype, two_streams):
             assert torch.equal(p.detach().reshape(-1).cpu(), ref_master[off:off + n].to(dtype)) or \
                 rel_err(p.detach().reshape(-1), ref_master[off:off + n]) <= 1e-2
         assert all(p.grad is None for p, *_ in b.param_view_specs)
+
+
+def _buckets_after(layers, xs, dev, dtype, streams, tasks_of):
+    store, ex, mbs, ubids = _make_executor(layers, xs, dev, dtype, streams)
+    out = ex.run(tasks_of(ubids), mbs)
+    torch.cuda.synchronize()
+    return out["losses"], {u: (store.buckets[u].flat_grads.clone(), store.buckets[u].flat_params.clone()) for u in store.buckets}
+
+
+def _assert_same_buckets(ref, got):
+    (l0, b0), (l1, b1) = ref, got
+    assert len(l0) == len(l1) and all(torch.equal(a, b) for a, b in zip(l0, l1))
+    for u in b0:
+        assert torch.equal(b0[u][0], b1[u][0]), f"gradient bucket {u}"
+        assert torch.equal(b0[u][1], b1[u][1]), f"parameter bucket {u}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_compute_stream_without_pack_stream(dev, dtype):
+    """Only a compute stream: backward and gradient pack share it, and it first waits for the
+    caller's stream, which produced the microbatches.  Same buckets, bit for bit, as on one stream."""
+    print(f"[case] compute stream only {dtype}", flush=True)
+    layers, xs = _init(3, dtype)
+    ref = _buckets_after(layers, xs, dev, dtype, False, lambda ubids: one_f_one_b(MB, ubids))
+    got = _buckets_after(layers, xs, dev, dtype, "compute only", lambda ubids: one_f_one_b(MB, ubids))
+    _assert_same_buckets(ref, got)
+
+
+@pytest.mark.parametrize("name, stages", [("schedule_pp1_1f1b_mb4.json", 1), ("schedule_pp1_zerobubble_mb4.json", 1),
+                                          ("schedule_pp2_zerobubble_mb4.json", 2)])
+def test_schedule_file_drives_the_executor(dev, name, stages):
+    """A schedule file in the reference's format (src/schedule.py:6-99) becomes the task list of
+    the one device and gives the same buckets as the hand-built 1F1B list."""
+    import os
+    from piper_amd.schedule import device_tasks, load_schedule_directives
+    print(f"[case] schedule file {name}", flush=True)
+    directives = load_schedule_directives(os.path.join(os.path.dirname(__file__), "golden", name))
+    layers, xs = _init(4, torch.float32)
+    ref = _buckets_after(layers, xs, dev, torch.float32, False, lambda ubids: one_f_one_b(MB, ubids))
+
+    def tasks_of(ubids):
+        stage_ubids = [list(ubids)] if stages == 1 else [[u] for u in ubids]
+        tasks = device_tasks(directives, stage_ubids)
+        assert tasks[-1].type is TaskType.UPD
+        return tasks
+
+    got = _buckets_after(layers, xs, dev, torch.float32, True, tasks_of)
+    # the losses come out in the order the last stage's backward passes run; every schedule here
+    # runs them by ascending microbatch
+    _assert_same_buckets(ref, got)
 
 
 def test_comm_tasks_are_noops_and_unknown_bucket_raises(dev):

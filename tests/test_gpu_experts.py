@@ -186,6 +186,40 @@ def test_reference_operator_bmm_experts(dev, counts_dtype):
     assert meta.shape == x.shape and meta.is_meta
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_bmm_experts_rows_past_the_last_expert_are_zero(dev, dtype):
+    """x has more rows than sum(num_tokens_per_expert): the reference returns zeros there
+    (`out = x.new_zeros`, qwen3_bmm_experts_patch.py:43) and no gradient flows into them.  Checked
+    against the oracle's restatement of the padded-bmm algorithm."""
+    print(f"[case] bmm_experts with unowned rows {dtype}", flush=True)
+    counts = [40, 0, 130, 5]
+    extra = 37
+    x, w1, w2, w3, dy, cnt = _make(11, counts, 256, 128, dtype)
+    g = torch.Generator().manual_seed(12)
+    x = torch.cat([x, torch.randn(extra, x.shape[1], generator=g).to(dtype)])
+    dy = torch.cat([dy, torch.randn(extra, dy.shape[1], generator=g).to(dtype)])
+    leaves = [t.float().requires_grad_(True) for t in (w1, w2, w3, x)]
+    y_ref = O.padded_bmm_experts(*leaves, cnt)
+    y_ref.backward(dy.float())
+    assert torch.count_nonzero(y_ref[sum(counts):]) == 0 and torch.count_nonzero(leaves[3].grad[sum(counts):]) == 0
+    F_.register_reference_op()
+    W1, W2, W3, X = (t.to(dev).requires_grad_(True) for t in (w1, w2, w3, x))
+    # poison the allocator's free blocks so that rows the kernels skip would show
+    junk = torch.full((x.shape[0] * 4, x.shape[1]), float("nan"), device=dev, dtype=dtype)
+    del junk
+    y = torch.ops.piper_artifact.bmm_experts(W1, W2, W3, X, cnt.to(dev))
+    tol = BF16_TOL if dtype == torch.bfloat16 else F32_TOL
+    assert torch.count_nonzero(y[sum(counts):]).item() == 0
+    assert rel_err(y, y_ref) <= tol
+    y.backward(dy.to(dev))
+    assert torch.count_nonzero(X.grad[sum(counts):]).item() == 0
+    assert rel_err(X.grad, leaves[3].grad) <= tol
+    for got, ref in zip((W1, W2, W3), leaves[:3]):
+        assert rel_err(got.grad, ref.grad) <= tol
+    with torch.no_grad():
+        assert torch.count_nonzero(torch.ops.piper_artifact.bmm_experts(W1, W2, W3, X, cnt.to(dev))[sum(counts):]).item() == 0
+
+
 def test_argument_errors(dev):
     z = torch.zeros(4, 8, device=dev, dtype=torch.bfloat16)
     w = torch.zeros(2, 16, 8, device=dev, dtype=torch.bfloat16)
