@@ -249,6 +249,30 @@ PK_API int pk_grouped_swiglu_wgrad_scaled(const void* d_out, const void* hs, con
                                    int accumulate, int64_t A, int64_t H, int64_t I, int64_t E,
                                    int dtype, pk_stream_t stream);
 
+/* The same pair with one operand of every weight-gradient GEMM K-contiguous (the fused region's
+ * path for bf16 with H % 256 == 0 and I % 256 == 0).  pk_grouped_swiglu_dgrad_dh_scaled_t writes
+ * d_g, d_u [A,I] as above and, instead of hs, the three transposed copies
+ *   d_gT, d_uT, hsT  [I][ldt]  (dtype), element (i, padded_start(e) + r) = row r of expert e,
+ *   padded_start(e) = (starts[e] & ~63) + 64*e; the columns from an expert's last row up to the next
+ *   multiple of 8 are zero, all other columns between experts are neither written nor read.
+ * ldt >= pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype) and a multiple of 64; that query returns
+ * 0 when the shape or dtype has no such path (use the entry points above then).
+ * pk_grouped_swiglu_wgrad_scaled_t computes the same d_w1, d_w2, d_w3 as
+ * pk_grouped_swiglu_wgrad_scaled from d_out, x (through row_map / row_map_div) and the transposed
+ * copies.  Both replace the autograd of qwen3_bmm_experts_patch.py:39-41 like the pair above. */
+PK_API int64_t pk_grouped_swiglu_transposed_ld(int64_t A, int64_t H, int64_t I, int64_t E, int dtype);
+PK_API int pk_grouped_swiglu_dgrad_dh_scaled_t(const void* d_out, const int32_t* row_map, int64_t row_map_div,
+                                        const float* scores, const void* w2, const void* g,
+                                        const void* u, const int32_t* starts, void* d_g, void* d_u,
+                                        void* d_gT, void* d_uT, void* hsT, int64_t ldt, float* d_scores,
+                                        void* workspace, int64_t workspace_bytes, int64_t A, int64_t H,
+                                        int64_t I, int64_t E, int dtype, pk_stream_t stream);
+PK_API int pk_grouped_swiglu_wgrad_scaled_t(const void* d_out, const void* hsT, const void* d_gT, const void* d_uT,
+                                     int64_t ldt, const void* x, const int32_t* row_map, int64_t row_map_div,
+                                     const int32_t* starts, const int32_t* expert_order, void* d_w1,
+                                     void* d_w2, void* d_w3, int accumulate, int64_t A, int64_t H,
+                                     int64_t I, int64_t E, int dtype, pk_stream_t stream);
+
 /* ------------------------------------------------------------- ZeRO bucket path */
 
 /* HOST function.  offsets[i] (in elements) of n tensors laid out back to back, each start

@@ -56,6 +56,13 @@ SIGNATURES = {
     "pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes": (_c_i64, [_c_i64, _c_i64]),
     "pk_grouped_swiglu_dgrad_dh_scaled": (_c_int, [_p, _p, _c_i64, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _c_i64,
                                                    _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
+    "pk_grouped_swiglu_transposed_ld": (_c_i64, [_c_i64, _c_i64, _c_i64, _c_i64, _c_int]),
+    # d_out row_map div scores w2 g u starts d_g d_u d_gT d_uT hsT ldt d_scores ws ws_bytes A H I E dtype stream
+    "pk_grouped_swiglu_dgrad_dh_scaled_t": (_c_int, [_p, _p, _c_i64, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _c_i64, _p,
+                                                     _p, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
+    # d_out hsT d_gT d_uT ldt x row_map div starts order d_w1 d_w2 d_w3 accumulate A H I E dtype stream
+    "pk_grouped_swiglu_wgrad_scaled_t": (_c_int, [_p, _p, _p, _p, _c_i64, _p, _p, _c_i64, _p, _p, _p, _p, _p, _c_int,
+                                                  _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
     "pk_bucket_plan": (_c_i64, [_p, _c_i64, _c_i64, _c_i64, _p]),
     "pk_bucket_pack": (_c_int, [_p, _p, _p, _c_i64, _c_int, _p, _c_int, _c_int, _p]),
     "pk_bucket_unpack": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_int, _p]),

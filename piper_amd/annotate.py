@@ -9,9 +9,6 @@ decide which region a call belongs to.
 """
 from __future__ import annotations
 
-import itertools
-from collections import Counter
-from typing import Iterator
 
 PP_TAG = "PP"
 EP_TAG = "EP"
@@ -44,12 +41,16 @@ class _Registry:
 
     def reset(self) -> None:
         self.active: list[dict] = []
-        self.per_name: Counter = Counter()
-        self.serial: Iterator[int] = itertools.count()
+        self.opened_per_name: dict[str, int] = {}
+        self.opened = 0
 
     def open(self, name: str) -> dict:
-        record = {"name": name, "index": self.per_name[name], "uid": next(self.serial)}
-        self.per_name[name] += 1
+        # plain ints and dicts only: the model's forward is captured by Dynamo with fullgraph=True,
+        # which has to trace through this bookkeeping
+        nth = self.opened_per_name.get(name, 0)
+        record = {"name": name, "index": nth, "uid": self.opened}
+        self.opened_per_name[name] = nth + 1
+        self.opened += 1
         self.active.append(record)
         return record
 

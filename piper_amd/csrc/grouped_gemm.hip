@@ -45,10 +45,15 @@ __device__ __forceinline__ int logical_block() {
 // Direct global->LDS load of 16 bytes per lane: lane l's bytes land at lds_base + 16*l.
 // Issued from inline asm so that the compiler does not serialise later LDS reads behind it;
 // completion is tracked by hand with vmcnt (wait_dma) followed by a workgroup barrier.
+// The statement sets M0 and uses it at once.  M0 cannot be named as clobbered (the compiler
+// treats it as reserved and rejects the promise to preserve it), and nothing else in these
+// kernels keeps a value in it: on gfx9 ordinary LDS accesses do not read M0, and the kernels
+// use no indirect register indexing, readlane with a register index excepted, which takes an
+// SGPR operand and not M0.
 __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off"
                :: "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr)
-               : "memory", "m0");
+               : "memory");
 }
 template <int N>
 __device__ __forceinline__ void wait_dma() {
@@ -383,6 +388,17 @@ __device__ __forceinline__ void sched_finish(SchedSlot* slot) {
   }
 }
 
+// Column at which expert e's rows start in a transposed ([width][ldt]) copy of an expert-sorted
+// operand: a multiple of 64 (128 bytes: the 32-row pieces that the producer stores and the 32-deep
+// k-tiles that the consumer loads then never straddle a 64-byte sector; with 16-byte alignment
+// the stores cost the producer 25 % of its time), computed from starts[e] alone.  Expert e owns
+// [padded_start(e), padded_start(e+1)), which holds its rows rounded up to a multiple of 8:
+// round_down64(a + n) + 64 > n.  ldt >= round_up64(A) + 64 * E holds every expert.
+constexpr int kTransposedAlign = 64;
+__host__ __device__ __forceinline__ int padded_start(int start, int e) {
+  return (start & ~(kTransposedAlign - 1)) + kTransposedAlign * e;
+}
+
 // Division of a non-negative int32 by a divisor fixed per launch without the ~25 instructions of
 // the general integer division: a shift for powers of two, otherwise multiply-high by
 // floor(2^(31+s)/d)+1 and shift by s-1 with s = ceil(log2 d) (exact for 0 <= n < 2^31).
@@ -429,6 +445,13 @@ struct RaggedMParams {
   const float* scores;   // SWIGLU_BWD_SCALED: score of sorted row r is scores[row_map[r]]
   float* ds_partial;     // SWIGLU_BWD_SCALED: [ldc / 64][total_rows] partial <unscaled d_h, h>
   int64_t total_rows;
+  // SWIGLU_BWD_SCALED, optional: the three outputs once more, transposed ([ldc][ldt], the routed
+  // rows contiguous) for the weight-gradient kernels that want a K-contiguous operand.  Expert e's
+  // rows start at column padded_start(e); columns up to the next multiple of 8 are zero.
+  bf16_t* T0;            // d_g^T
+  bf16_t* T1;            // d_u^T
+  bf16_t* T2;            // (score * h)^T
+  int64_t ldt;
   SchedSlot* sched;      // this launch's counters
 };
 
@@ -444,8 +467,9 @@ struct Stage32 {
     *reinterpret_cast<u32x2_t*>(buf + row * ROWB + ((((col >> 3) ^ row) & (CH - 1)) << 4) + (col & 7) * 2) = v;
   }
   // rows [0, nrows) go to dst[r * ldc + 0..COLS); returns the number of store instructions
-  // the wave issued (nrows is wave-uniform)
-  template <bool ACC>
+  // the wave issued (nrows is wave-uniform).  STREAM: nontemporal stores, for results that neither
+  // this nor the next kernels read (weight gradients).
+  template <bool ACC, bool STREAM = false>
   __device__ static __forceinline__ int flush(const char* buf, bf16_t* dst, int64_t ldc, int nrows) {
     constexpr int RPP = 64 / CH, NP = 32 / RPP;
     const int lane = threadIdx.x & 63;
@@ -469,10 +493,42 @@ struct Stage32 {
           for (int t = 0; t < 8; ++t) sum[t] = (bf16_t)((float)a[t] + (float)o[t]);
           v[q] = __builtin_bit_cast(u32x4_t, sum);
         }
-        *g = v[q];
+        if (STREAM) __builtin_nontemporal_store(v[q], g);
+        else *g = v[q];
       }
     }
     return nrows >= 32 ? NP : nrows <= 0 ? 0 : (nrows + RPP - 1) / RPP;
+  }
+  // The staged tile transposed: element (r, c) goes to dstT[c * ldt + r], rows in groups of 8
+  // (16 bytes per lane): the groups that start below nrows are written, so the caller stages zeros
+  // in rows nrows..31 when the columns up to the next multiple of 8 must come out as zeros.  dstT
+  // + multiples of ldt must be 16-byte aligned.  The transposing LDS read hands a lane 4
+  // consecutive rows of one column: within 16 lanes, lane i points at row i/4, columns 4*(i%4)..+3
+  // and receives rows 0..3 of column i.  One store instruction covers 16 columns x 32 rows: the
+  // four 16-lane groups take the four 8-row groups, so each destination row receives 64
+  // contiguous bytes per instruction.  Returns the number of store instructions issued.
+  __device__ static __forceinline__ int flush_t(const char* buf, bf16_t* dstT, int64_t ldt, int nrows) {
+    static_assert(COLS == 64, "four passes of 16 columns");
+    const int lane = threadIdx.x & 63;
+    const int i = lane & 15, grp = lane >> 4;
+    const int r0 = 8 * grp + (i >> 2), r1 = r0 + 4;
+    typedef short shortx8_t __attribute__((ext_vector_type(8)));
+    u32x4_t v[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {                    // columns 16q .. 16q+15
+      const int col = 16 * q + 4 * (i & 3);          // first of the 4 columns this lane points at
+      const char* p0 = buf + r0 * ROWB + ((((col >> 3) ^ r0) & (CH - 1)) << 4) + (col & 7) * 2;
+      const char* p1 = buf + r1 * ROWB + ((((col >> 3) ^ r1) & (CH - 1)) << 4) + (col & 7) * 2;
+      const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) shortx4_t*)(p0));
+      const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) shortx4_t*)(p1));
+      v[q] = __builtin_bit_cast(u32x4_t, (shortx8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+    if (8 * grp < nrows) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<u32x4_t*>(dstT + (int64_t)(16 * q + i) * ldt + 8 * grp) = v[q];
+    }
+    return nrows > 0 ? 4 : 0;
   }
 };
 
@@ -612,6 +668,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
 
   struct Unit {
     int row0, rows, nt;
+    int tcol;            // column of row0 in the transposed outputs
     int64_t b_base;
     int64_t a_off[LA];
   };
@@ -622,6 +679,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     t.row0 = s0 + mt * BM;
     t.rows = min(BM, s1 - t.row0);
     t.nt = nt;
+    t.tcol = padded_start(s0, e) + mt * BM;
     t.b_base = (int64_t)e * p.strideB + (B_KC ? (int64_t)nt * BN_OUT * p.ldb : (int64_t)nt * BN);
 #pragma unroll
     for (int i = 0; i < LA; ++i) {
@@ -683,8 +741,15 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
 #pragma unroll
   for (int s = 0; s < NS - 1; ++s) issue_tile(cur_u, s, s);
 
+  Unit ld_u = cur_u;    // the unit whose k-tiles are being requested: the current one or, chained, the next
   for (;;) {
     int unit_next = -1;
+    // chained: the k-loop goes on requesting k-tiles past the end of this unit -- the first NS-1
+    // of the next unit -- in the slots where it would otherwise request blocks of zeros.  The next
+    // unit's operands are then in LDS when this unit's epilogue ends, and the epilogue's stores do
+    // not stand between those requests and the first MFMA of the next unit.
+    bool chained = false;
+    ld_u = cur_u;
     const bool wave_has_rows = wm * WTM < cur_u.rows;   // waves whose row slice is empty skip the math
 
     floatx16_t acc[TM][TN];
@@ -715,18 +780,22 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
       if (kt == 1) {                    // the box was written before this k-tile's barrier
         unit_next = __builtin_amdgcn_readfirstlane(sched_box[par ^ 1]);
         if (unit_next >= 0) setup(nxt_u, unit_next);
+        chained = unit_next >= 0 && nkt >= NS + 1;
       }
+      const int slot = kt + NS - 1;                                   // the k-tile slot requested during this tile
+      const bool of_next = chained && slot >= nkt;
+      if (of_next && slot == nkt) ld_u = nxt_u;
       const int tgt = cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1;   // stage of k-tile kt-1 = kt+NS-1
-      issue_setup(kt + NS - 1, tgt);
-      is_real = kt + NS - 1 < nkt;
+      issue_setup(of_next ? slot - nkt : slot, tgt);
+      is_real = of_next || slot < nkt;
       const char* st = smem + cur * STAGE;
       const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
       if (wave_has_rows) {
         mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN,
-                                                     f0, acc, [&](int piece) { issue_piece(cur_u, piece); });
+                                                     f0, acc, [&](int piece) { issue_piece(ld_u, piece); });
       } else {
 #pragma unroll
-        for (int i = 0; i < L; ++i) issue_piece(cur_u, i);
+        for (int i = 0; i < L; ++i) issue_piece(ld_u, i);
       }
       cur = cur + 1 == NS ? 0 : cur + 1;
     }
@@ -736,7 +805,11 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     // one round trip on one wave, not a drain of stores
     if (has_next && tid == 0) grab = sched_grab(p.sched, xcd);
 
+    // the next unit's first k-tiles, unless the k-loop has requested them already (then every
+    // store of this epilogue is younger than they are)
+    if (chained) st_after = 0;
     auto prefetch_next = [&]() {
+      if (chained) return;
       st_after = 0;
       if (has_next) {
 #pragma unroll
@@ -749,6 +822,44 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     const int lrow = lane & 31, lq = 4 * (lane >> 5);
     const int64_t grow0 = (int64_t)(cur_u.row0 + wm * WTM) * p.ldc;
     const int64_t gcol0 = (int64_t)cur_u.nt * BN_OUT + wn * OUT_COLS;
+    // SwiGLU backward: the epilogue reads g and u (and, scaled, the row's combine score through the
+    // row map).  Each of these is a round trip to HBM, so they are requested in batches: all scores
+    // first, then the vectors of JB column tiles of a 32-row chunk at once (a whole chunk where the
+    // registers allow it).  One vector at a time, as the compiler orders the loop below on its
+    // own, costs a wave about 2,000 cycles per vector: a quarter of a 128-row unit's time at 4,096
+    // tokens.
+    constexpr int JB = !BWD ? 1 : (TM <= 2 ? TN : 1);     // column tiles per batch
+    u32x2_t graw[JB][4], uraw[JB][4];
+    float sc_chunk[BWD ? TM : 1];
+    auto load_gu = [&](int i, int j0) {
+      const int crows = min(32, cur_u.rows - wm * WTM - 32 * i);
+      if (crows <= 0) return;
+      const int rr = lrow < crows ? lrow : crows - 1;
+      const int64_t goff = grow0 + (int64_t)(32 * i) * p.ldc + gcol0 + (int64_t)rr * p.ldc + lq;
+#pragma unroll
+      for (int j = 0; j < JB; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          graw[j][q] = *reinterpret_cast<const u32x2_t*>(p.Gin + goff + 32 * (j0 + j) + 8 * q);
+          uraw[j][q] = *reinterpret_cast<const u32x2_t*>(p.Uin + goff + 32 * (j0 + j) + 8 * q);
+        }
+    };
+    if constexpr (BWD) {
+      if constexpr (SCALED) {
+        int slot[TM];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int crows = min(32, cur_u.rows - wm * WTM - 32 * i);
+          const int rr = lrow < crows ? lrow : (crows > 0 ? crows - 1 : 0);
+          slot[i] = crows > 0 ? p.row_map[cur_u.row0 + wm * WTM + 32 * i + rr] : 0;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) sc_chunk[i] = p.scores[slot[i]];
+      } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) sc_chunk[i] = 1.f;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int crows = min(32, cur_u.rows - wm * WTM - 32 * i);   // valid rows of this chunk
@@ -794,19 +905,20 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
         u32x2_t dg[TN][4], du[TN][4], hs[SCALED ? TN : 1][4];
         float ds = 0.f;
         if (crows > 0) {
-          const int rr = lrow < crows ? lrow : crows - 1;
-          float sc = 1.f;
-          if (SCALED) sc = p.scores[p.row_map[cur_u.row0 + wm * WTM + 32 * i + rr]];
+          const float sc = sc_chunk[i];
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
+          for (int j = 0; j < TN; ++j) {
+            if (j % JB == 0) {
+              load_gu(i, j);
+              __builtin_amdgcn_sched_barrier(0);    // keep the batch together, ahead of the arithmetic
+            }
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-              const int64_t off = goff + (int64_t)rr * p.ldc + 32 * j + 8 * q + lq;
               float dh[4], g[4], u[4], og[4], ou[4], oh[4];
               // d_h is rounded to bf16 first, like the output of the reference's batched matmul
               unpack4(pack4(sc * acc[i][j][4 * q], sc * acc[i][j][4 * q + 1], sc * acc[i][j][4 * q + 2], sc * acc[i][j][4 * q + 3]), dh);
-              unpack4(*reinterpret_cast<const u32x2_t*>(p.Gin + off), g);
-              unpack4(*reinterpret_cast<const u32x2_t*>(p.Uin + off), u);
+              unpack4(graw[j % JB][q], g);
+              unpack4(uraw[j % JB][q], u);
 #pragma unroll
               for (int t = 0; t < 4; ++t) {
                 const float sg = 1.f / (1.f + __expf(-g[t]));
@@ -822,6 +934,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
               du[j][q] = pack4(ou[0], ou[1], ou[2], ou[3]);
               if (SCALED) hs[j][q] = pack4(oh[0], oh[1], oh[2], oh[3]);
             }
+          }
         }
         // the loads above must have returned first: a load behind the prefetch waits for all of it
         __builtin_amdgcn_sched_barrier(0);
@@ -834,15 +947,27 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
               p.ds_partial[(int64_t)((cur_u.nt * BN + wn * WTN) >> 6) * p.total_rows + cur_u.row0 + wm * WTM + 32 * i + lrow] = ds;
             st_after += 1;
           }
+          const bool transposed = SCALED && p.T0 != nullptr;
+          const bool live = lrow < crows;      // the transposed copies want zeros in the rows past the end
+          const u32x2_t zero2 = {0u, 0u};
 #pragma unroll
           for (int which = 0; which < (SCALED ? 3 : 2); ++which) {
+            bf16_t* const out = which == 0 ? p.O0 : which == 1 ? p.O1 : p.O2;
+            if (which == 2 && !out && !transposed) continue;
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
-              for (int q = 0; q < 4; ++q)
-                St::put(sbuf, lrow, 32 * j + 8 * q + lq, which == 0 ? dg[j][q] : which == 1 ? du[j][q] : hs[SCALED ? j : 0][q]);
+              for (int q = 0; q < 4; ++q) {
+                const u32x2_t v = which == 0 ? dg[j][q] : which == 1 ? du[j][q] : hs[SCALED ? j : 0][q];
+                St::put(sbuf, lrow, 32 * j + 8 * q + lq, (transposed && !live) ? zero2 : v);
+              }
             wave_lds_fence();
-            st_after += St::template flush<false>(sbuf, (which == 0 ? p.O0 : which == 1 ? p.O1 : p.O2) + goff, p.ldc, crows);
+            if (out) st_after += St::template flush<false>(sbuf, out + goff, p.ldc, crows);
+            if constexpr (SCALED) {
+              if (transposed)
+                st_after += St::flush_t(sbuf, (which == 0 ? p.T0 : which == 1 ? p.T1 : p.T2) + gcol0 * p.ldt + (cur_u.tcol + wm * WTM + 32 * i),
+                                        p.ldt, crows);
+            }
             wave_lds_fence();
           }
         }
@@ -1069,6 +1194,329 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
   wave_lds_fence();
   if (p.accumulate) St::template flush<WTM, true>(sbuf, C, q.N, WTM);
   else St::template flush<WTM, false>(sbuf, C, q.N, WTM);
+}
+
+// ---- weight gradient with one K-contiguous operand, persistent workgroups.
+// C[e][M,N] (+)= sum over the rows r of expert e of  m-side[r, m] * n-side[r, n], where one side comes
+// from a transposed copy ("T": [width][ldt], the routed rows contiguous, expert e at column
+// padded_start(e), written by the scaled SwiGLU backward) and the other side from rows gathered
+// through the row map ("R": x or d_out).  Against wgrad_kernel: the T operand is read with
+// ds_read_b128 instead of the transposing read (the LDS read rate bounds a k-loop whose operands
+// both need it), a workgroup walks units taken from the per-XCD counters, requests the first
+// k-tiles of its next unit before the epilogue of the current one, and its stores do not hold up
+// the next unit's loads.  A_KC: T is the m side (d_w1 = d_g^T x, d_w3 = d_u^T x); otherwise T is the
+// n side (d_w2 = d_out^T (score h)).  The wave grid puts the wider wave-tile side on T.
+struct WgradKcProblem {
+  const bf16_t* T;
+  const bf16_t* R;
+  bf16_t* C;
+};
+struct WgradKcParams {
+  WgradKcProblem prob[2];
+  int64_t ldt, ldr;
+  const int32_t* row_map;    // sorted row -> flat slot; R row = slot / map_div
+  FastDiv map_div;
+  const int32_t* starts;
+  const int32_t* order;      // optional [E]: experts by descending row count
+  int32_t E, nprob;
+  int32_t M, N;              // output per expert (multiples of the block tile)
+  int32_t total_rows;        // A: entries of the row map
+  int32_t accumulate;
+  SchedSlot* sched;
+};
+
+template <int BM, int BN, int BK, int WMW, int WNW, int NS, bool A_KC, bool DYNAMIC>
+__global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcParams p) {
+  constexpr bool B_KC = !A_KC;
+  constexpr int NW = WMW * WNW, NTHREADS = 64 * NW;
+  constexpr int WTM = BM / WMW, WTN = BN / WNW, TM = WTM / 32, TN = WTN / 32;
+  constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE = A_BYTES + B_BYTES;
+  constexpr int KC_ROWS = A_KC ? BM : BN, MN_COLS = A_KC ? BN : BM;
+  constexpr int KC_OFF = A_KC ? 0 : A_BYTES, MN_OFF = A_KC ? A_BYTES : 0;
+  constexpr int LKC = KC_ROWS * BK * 2 / (NTHREADS * 16), LMN = MN_COLS * BK * 2 / (NTHREADS * 16), L = LKC + LMN;
+  constexpr int MN_CPR = MN_COLS / 8, MN_RPI = 64 / MN_CPR, NR = LMN * MN_RPI;
+  static_assert(LKC >= 1 && LMN >= 1 && MN_RPI >= 1, "tile too small for the wave grid");
+  static_assert(WTN % 64 == 0, "the epilogue stages 64 columns at a time");
+  static_assert(NS >= 3, "the k-loop reads the next tile's first fragments one tile ahead");
+  using St = Stage32<64>;
+  constexpr int RING = NS * STAGE;
+  static_assert(RING + NW * St::BYTES <= 160 * 1024, "LDS budget");
+  __shared__ __attribute__((aligned(1024))) char smem[RING + NW * St::BYTES];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WNW, wn = wave % WNW;
+  char* const sbuf = smem + RING + wave * St::BYTES;
+  const const_i32_ptr starts = as_const(p.starts);
+  const const_i32_ptr row_map = as_const(p.row_map);
+  const const_i32_ptr order = as_const(p.order);
+  const int n_tiles = p.N / BN;
+  const int tiles = (p.M / BM) * n_tiles;
+  const int per_expert = tiles * p.nprob;
+  const int total = p.E * per_expert;
+  const int64_t ldt = p.ldt, ldr = p.ldr;
+
+  // ---- which units this workgroup runs.
+  // DYNAMIC: from the per-XCD counters, as in ragged_m_kernel (balances the very uneven experts of
+  // skewed routing); the next unit is published through LDS, double buffered, in the first bytes
+  // of wave 0's staging buffer (idle while a k-loop runs).
+  // Otherwise statically: round r gives XCD x the units [(r*8 + x) * G8, +G8), one per workgroup
+  // of that XCD (G8 workgroups per XCD), so the workgroups of an XCD work on neighbouring tiles of
+  // the same experts at the same time; the experts come in descending row count (p.order), so the
+  // units of one round cost about the same.  No atomics, no hand-over through LDS: a few per cent
+  // faster when every expert has a few hundred rows.
+  int* const sched_box = reinterpret_cast<int*>(smem + RING);
+  const int xcd = blockIdx.x % NXCD, G8 = gridDim.x / NXCD;
+  auto unit_at = [&](int r) {
+    const int u = (r * NXCD + xcd) * G8 + (int)(blockIdx.x / NXCD);
+    return u < total ? u : -1;
+  };
+  unsigned grab = 0;
+  int par = 0, round = 0;
+  int unit;
+  if constexpr (DYNAMIC) {
+    if (tid == 0) {
+      const int first = sched_resolve(p.sched, xcd, sched_grab(p.sched, xcd), total);
+      sched_box[0] = first;
+      if (first >= 0) grab = sched_grab(p.sched, xcd);
+    }
+    __syncthreads();
+    unit = __builtin_amdgcn_readfirstlane(sched_box[0]);
+    if (unit < 0) {
+      if (tid == 0) sched_finish(p.sched);
+      return;
+    }
+  } else {
+    unit = unit_at(0);
+    if (unit < 0) return;
+  }
+
+  // ---- lane constants of the loaders
+  int64_t kc_loff[LKC];   // element offset of this lane's 16 bytes inside a T tile: row * ldt + k
+  int kc_k[LKC];
+#pragma unroll
+  for (int i = 0; i < LKC; ++i) {
+    int r;
+    kc_slot<BK>(wave * LKC + i, lane, r, kc_k[i]);
+    kc_loff[i] = (int64_t)r * ldt + kc_k[i];
+  }
+  int mn_cofs[LMN], mn_krow[LMN];          // column offset and k-row (inside a tile) of this lane's 16 bytes
+#pragma unroll
+  for (int i = 0; i < LMN; ++i) mn_slot<MN_COLS>(wave * LMN + i, lane, mn_krow[i], mn_cofs[i]);
+  const int mn_rsel = lane / MN_CPR;       // which of the MN_RPI rows of a load this lane fetches
+
+  struct Unit {
+    int e, q, mt, nt;
+    int s0, rows, nkt, kcols;    // first sorted row, row count, k-tiles, rows rounded up to 8
+    const bf16_t* t_base;        // T + first tile row * ldt + padded_start(e)
+    const bf16_t* r_base;        // R + first tile column
+  };
+  auto setup = [&](Unit& t, int un) {
+    const int rank = un / per_expert;
+    const int rem = un - rank * per_expert;
+    t.q = rem / tiles;
+    const int tt = rem - t.q * tiles;
+    t.mt = tt / n_tiles;
+    t.nt = tt - t.mt * n_tiles;
+    t.e = p.order ? order[rank] : rank;
+    t.s0 = starts[t.e];
+    t.rows = starts[t.e + 1] - t.s0;
+    t.nkt = (t.rows + BK - 1) / BK;
+    t.kcols = (t.rows + 7) & ~7;
+    const WgradKcProblem& q = p.prob[t.q];
+    t.t_base = q.T + (int64_t)(A_KC ? t.mt * BM : t.nt * BN) * ldt + padded_start(t.s0, t.e);
+    t.r_base = q.R + (A_KC ? t.nt * BN : t.mt * BM);
+  };
+  // Flat slots (row map entries) of the R rows of k-tile kt, wave-uniform, fetched with scalar
+  // loads one tile before they are needed.  No branch and no arithmetic here: rows past the
+  // expert's end read a clamped index and are masked per lane when the load is issued, and the
+  // division by the map divisor happens per lane as well (a chain of scalar instructions per row
+  // -- compare, select, divide, 64-bit multiply -- cost this loop 600 of its 2,400 cycles per k-tile).
+  int rows_n[NR];
+  auto fetch_rows = [&](const Unit& t, int kt) {
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      // load i / MN_RPI of this wave, row i % MN_RPI of the load
+      const int k = kt * BK + (wave * LMN + i / MN_RPI) * MN_RPI + i % MN_RPI;
+      rows_n[i] = row_map[min(t.s0 + k, p.total_rows - 1)];
+    }
+  };
+  // The unit whose tiles are being requested (the current one, or, towards the end of a k-loop,
+  // the next one), reduced to what the loader needs.
+  struct LoadSrc {
+    int rows, nkt, kcols;
+    const bf16_t* t_base;
+    const bf16_t* r_base;
+  };
+  auto load_src = [](const Unit& t) { return LoadSrc{t.rows, t.nkt, t.kcols, t.t_base, t.r_base}; };
+  LoadSrc ld;
+  uint32_t is_kc = 0, is_mn = 0;
+  int is_k0 = 0;
+  bool is_real = true;
+  auto issue_setup = [&](int kt, int stage) {
+    is_k0 = kt * BK;
+    is_real = kt < ld.nkt;
+    is_kc = lds_addr(smem + stage * STAGE + KC_OFF) + (wave * LKC) * 1024;
+    is_mn = lds_addr(smem + stage * STAGE + MN_OFF) + (wave * LMN) * 1024;
+  };
+  // Every k-tile slot issues its L loads; what lies past the expert's rows reads a block of zeros.
+  auto issue_piece = [&](int piece) {
+    if (piece < LKC) {
+      const bool ok = is_real && (is_k0 + kc_k[piece] < ld.kcols);
+      const void* src = ld.t_base + kc_loff[piece] + is_k0;
+      dma16(ok ? src : (const void*)g_zero16, is_kc + piece * 1024);
+    } else {
+      const int i = piece - LKC;
+      int slot = rows_n[i * MN_RPI];
+#pragma unroll
+      for (int r = 1; r < MN_RPI; ++r) slot = mn_rsel == r ? rows_n[i * MN_RPI + r] : slot;
+      const bool ok = is_real && (is_k0 + mn_krow[i] < ld.rows);
+      const void* src = ld.r_base + (int64_t)fastdiv(slot, p.map_div) * ldr + mn_cofs[i];
+      dma16(ok ? src : (const void*)g_zero16, is_mn + i * 1024);
+    }
+  };
+  // the first NS-1 k-tiles of unit t into the stages from `first_stage` on
+  auto issue_prologue = [&](const Unit& t, int first_stage) {
+    ld = load_src(t);
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s) {
+      issue_setup(s, first_stage + s >= NS ? first_stage + s - NS : first_stage + s);
+      fetch_rows(t, s);
+#pragma unroll
+      for (int i = 0; i < L; ++i) issue_piece(i);
+    }
+  };
+
+  int st_after = 0;     // stores this wave issued after the latest k-tile request
+  Unit cur_u, nxt_u;
+  setup(cur_u, unit);
+  nxt_u = cur_u;
+  int cur = 0;          // ring stage of k-tile 0 of the current unit
+  issue_prologue(cur_u, 0);
+
+  for (;;) {
+    int unit_next = -1;
+    bool resolved = false;
+    // chained: the k-loop goes on requesting tiles past the end of this unit -- the first NS-1 of
+    // the next unit -- where it would otherwise request blocks of zeros, so the next unit's
+    // operands are in LDS when this unit's epilogue ends and the stores of the epilogue do not
+    // stand between the requests and the first MFMA.  Needs the next unit to be known NS tiles
+    // before the end (its row map entries are fetched one tile ahead of the request).
+    bool chained = false;
+    const int nkt = cur_u.nkt;
+    ld = load_src(cur_u);
+    floatx16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    if (nkt > 0) {
+      wait_vm_le((NS - 2) * L + st_after);     // k-tile 0 has landed: only younger operations are in flight
+      block_barrier();
+      Frags<TM, TN> f0;
+      load_frags<BK, TM, TN, A_KC, B_KC, BM, BN>(f0, smem + cur * STAGE, smem + cur * STAGE + A_BYTES, wm * WTM, wn * WTN, 0, lane);
+      fetch_rows(cur_u, NS - 1);
+      for (int kt = 0; kt < nkt; ++kt) {
+        if (kt == 0) wait_vm_le((NS - 3) * L + st_after);
+        else wait_dma<(NS - 3) * L>();
+        block_barrier();   // tile kt+1 is in LDS for everyone; everyone is done reading tile kt-1
+        if constexpr (DYNAMIC) {
+          if (kt == 0 && tid == 0) lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, total));
+          if (kt == 1) {
+            unit_next = __builtin_amdgcn_readfirstlane(sched_box[par ^ 1]);
+            if (unit_next >= 0) setup(nxt_u, unit_next);
+            resolved = true;
+            chained = unit_next >= 0 && nkt >= NS + 1;
+          }
+        } else {
+          if (kt == 0) {     // the scalar loads of the next unit's description run under this tile's MFMAs
+            unit_next = unit_at(round + 1);
+            if (unit_next >= 0) setup(nxt_u, unit_next);
+            resolved = true;
+            chained = unit_next >= 0 && nkt >= NS + 1;
+          }
+        }
+        const int slot = kt + NS - 1;                  // the k-tile slot requested during this tile
+        const bool of_next = chained && slot >= nkt;
+        if (of_next && slot == nkt) ld = load_src(nxt_u);
+        const int tgt = cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1;
+        issue_setup(of_next ? slot - nkt : slot, tgt);
+        const char* st = smem + cur * STAGE;
+        const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
+        mma_ktile<BK, TM, TN, A_KC, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN, f0, acc,
+                                                     [&](int piece) { issue_piece(piece); });
+        // row map entries of the slot after this one
+        if (chained && slot + 1 >= nkt) fetch_rows(nxt_u, slot + 1 - nkt);
+        else fetch_rows(cur_u, slot + 1);
+        cur = cur + 1 == NS ? 0 : cur + 1;
+      }
+    }
+    block_barrier();   // every wave has finished its fragment reads: the whole ring is free
+    if constexpr (DYNAMIC) {
+      if (!resolved) {   // fewer than two k-tiles: the next unit is settled here instead of in the k-loop
+        if (nkt == 0) {
+          if (tid == 0) lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, total));
+          block_barrier();
+        }
+        unit_next = __builtin_amdgcn_readfirstlane(sched_box[par ^ 1]);
+        if (unit_next >= 0) setup(nxt_u, unit_next);
+        block_barrier();   // the box lies in wave 0's staging buffer, which the epilogue is about to use
+      }
+    } else {
+      if (!resolved) {   // an expert without rows has no k-loop
+        unit_next = unit_at(round + 1);
+        if (unit_next >= 0) setup(nxt_u, unit_next);
+      }
+    }
+    const bool has_next = unit_next >= 0;
+    if constexpr (DYNAMIC) {
+      if (has_next && tid == 0) grab = sched_grab(p.sched, xcd);
+    }
+
+    // the next unit's first tiles, unless the k-loop has requested them already
+    auto prefetch_next = [&]() {
+      st_after = 0;
+      if (has_next && !chained) issue_prologue(nxt_u, cur);
+    };
+    // an accumulating epilogue reads the old gradients, and a wave waits for a load only together
+    // with everything it requested before it: there the requests go behind the epilogue
+    if (!p.accumulate || chained) prefetch_next();
+
+    if (!(p.accumulate && nkt == 0)) {
+      const WgradKcProblem& q = p.prob[cur_u.q];
+      bf16_t* const C = q.C + (int64_t)cur_u.e * p.M * p.N + (int64_t)(cur_u.mt * BM + wm * WTM) * p.N + cur_u.nt * BN + wn * WTN;
+      const int lrow = lane & 31, lq = 4 * (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int jh = 0; jh < TN; jh += 2) {
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd)
+              St::put(sbuf, lrow, 32 * jj + 8 * qd + lq,
+                      pack4(acc[i][jh + jj][4 * qd], acc[i][jh + jj][4 * qd + 1], acc[i][jh + jj][4 * qd + 2], acc[i][jh + jj][4 * qd + 3]));
+          wave_lds_fence();
+          bf16_t* const dst = C + (int64_t)(32 * i) * p.N + 32 * jh;
+          if (p.accumulate) St::template flush<true, true>(sbuf, dst, p.N, 32);
+          else st_after += St::template flush<false, true>(sbuf, dst, p.N, 32);
+          wave_lds_fence();
+        }
+    }
+    if (p.accumulate && !chained) prefetch_next();
+    if (!has_next) break;
+    cur_u = nxt_u;
+    unit = unit_next;
+    par ^= 1;
+    ++round;
+  }
+  wait_dma<0>();   // the zero loads of the last k-tiles must not land in LDS that a later workgroup owns
+  if constexpr (DYNAMIC) {
+    if (tid == 0) sched_finish(p.sched);
+  }
 }
 
 inline int round_up_xcd(int64_t n) { return (int)(pk_ceil_div(n, NXCD) * NXCD); }
@@ -1380,17 +1828,37 @@ int64_t pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes(int64_t A, int64_t I) 
   return pk_ceil_div(I, 64) * A * (int64_t)sizeof(float);
 }
 
-int pk_grouped_swiglu_dgrad_dh_scaled(const void* d_out, const int32_t* row_map, int64_t row_map_div,
-                                      const float* scores, const void* w2, const void* g,
-                                      const void* u, const int32_t* starts, void* d_g, void* d_u,
-                                      void* hs, float* d_scores, void* workspace,
-                                      int64_t workspace_bytes, int64_t A, int64_t H, int64_t I,
-                                      int64_t E, int dtype, pk_stream_t stream) {
+int64_t pk_grouped_swiglu_transposed_ld(int64_t A, int64_t H, int64_t I, int64_t E, int dtype) {
+  if (A < 0 || H <= 0 || I <= 0 || E <= 0) return PK_ERR_ARG;
+  if (dtype != PK_BF16 || H % 256 != 0 || I % 256 != 0 || E > PK_MAX_EXPERTS || A + (int64_t)mf::kTransposedAlign * E > 0x7fffff00ll) return 0;
+  // an odd multiple of 256 bytes: consecutive rows of a transposed copy then start in different
+  // 256-byte phases of a 4 KiB period, so the 16 rows that one store (or the 256 rows that one
+  // tile load) touches at the same column do not all map to the same memory channel
+  int64_t units = ((A + mf::kTransposedAlign - 1) / mf::kTransposedAlign + E + 1) / 2;
+  if (units % 2 == 0) ++units;
+  return units * 2 * mf::kTransposedAlign;
+}
+
+// transposed outputs (d_gT, d_uT, hsT: [I][ldt]) are optional; with them hs itself may be NULL
+static int dgrad_dh_scaled_impl(const void* d_out, const int32_t* row_map, int64_t row_map_div,
+                                const float* scores, const void* w2, const void* g,
+                                const void* u, const int32_t* starts, void* d_g, void* d_u,
+                                void* hs, void* d_gT, void* d_uT, void* hsT, int64_t ldt, float* d_scores,
+                                void* workspace, int64_t workspace_bytes, int64_t A, int64_t H, int64_t I,
+                                int64_t E, int dtype, pk_stream_t stream) {
   int rc = check_common(A, H, I, E, dtype);
   if (rc) return rc;
   if (A == 0) return PK_OK;
-  if (!d_out || !row_map || row_map_div <= 0 || row_map_div > 0x7fffffffll || !scores || !w2 || !g || !u || !starts || !d_g || !d_u || !hs || !d_scores)
+  const bool transposed = d_gT != nullptr;
+  if (!d_out || !row_map || row_map_div <= 0 || row_map_div > 0x7fffffffll || !scores || !w2 || !g || !u || !starts || !d_g || !d_u || !d_scores)
     return PK_ERR_ARG;
+  if (!hs && !transposed) return PK_ERR_ARG;
+  if (transposed) {
+    const int64_t need = pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype);
+    if (need <= 0) return PK_ERR_SHAPE;
+    if (!d_uT || !hsT || ldt < need || ldt % 64 != 0) return PK_ERR_ARG;
+    if (!all_aligned16({d_out, w2, g, u, d_g, d_u, hs, d_gT, d_uT, hsT})) return PK_ERR_ALIGN;
+  }
   hipStream_t s = (hipStream_t)stream;
   const bool simt = dtype == PK_F32 || !mfma_shape_ok(H, I) || !all_aligned16({d_out, w2, g, u, d_g, d_u, hs});
   if (simt) {
@@ -1417,6 +1885,7 @@ int pk_grouped_swiglu_dgrad_dh_scaled(const void* d_out, const int32_t* row_map,
   p.starts = starts; p.E = (int32_t)E; p.Kseg = (int32_t)H; p.nseg = 1;
   p.Gin = (const bf16_t*)g; p.Uin = (const bf16_t*)u;
   p.O0 = (bf16_t*)d_g; p.O1 = (bf16_t*)d_u; p.O2 = (bf16_t*)hs; p.ldc = I;
+  p.T0 = (bf16_t*)d_gT; p.T1 = (bf16_t*)d_uT; p.T2 = (bf16_t*)hsT; p.ldt = ldt;
   p.scores = scores; p.ds_partial = (float*)workspace; p.total_rows = A;
   rc = launch_rm<false, mf::EPI_SWIGLU_BWD_SCALED>(p, A, I, pk_timing::K_SWIGLU_DGRAD_DH, s);
   if (rc) return rc;
@@ -1424,6 +1893,28 @@ int pk_grouped_swiglu_dgrad_dh_scaled(const void* d_out, const int32_t* row_map,
                     (const float*)workspace, (int)(I / 64), A, row_map, d_scores);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
+}
+
+int pk_grouped_swiglu_dgrad_dh_scaled(const void* d_out, const int32_t* row_map, int64_t row_map_div,
+                                      const float* scores, const void* w2, const void* g,
+                                      const void* u, const int32_t* starts, void* d_g, void* d_u,
+                                      void* hs, float* d_scores, void* workspace,
+                                      int64_t workspace_bytes, int64_t A, int64_t H, int64_t I,
+                                      int64_t E, int dtype, pk_stream_t stream) {
+  if (A > 0 && !hs) return PK_ERR_ARG;
+  return dgrad_dh_scaled_impl(d_out, row_map, row_map_div, scores, w2, g, u, starts, d_g, d_u, hs, nullptr, nullptr,
+                              nullptr, 0, d_scores, workspace, workspace_bytes, A, H, I, E, dtype, stream);
+}
+
+int pk_grouped_swiglu_dgrad_dh_scaled_t(const void* d_out, const int32_t* row_map, int64_t row_map_div,
+                                        const float* scores, const void* w2, const void* g,
+                                        const void* u, const int32_t* starts, void* d_g, void* d_u,
+                                        void* d_gT, void* d_uT, void* hsT, int64_t ldt, float* d_scores,
+                                        void* workspace, int64_t workspace_bytes, int64_t A, int64_t H,
+                                        int64_t I, int64_t E, int dtype, pk_stream_t stream) {
+  if (A > 0 && (!d_gT || !d_uT || !hsT)) return PK_ERR_ARG;
+  return dgrad_dh_scaled_impl(d_out, row_map, row_map_div, scores, w2, g, u, starts, d_g, d_u, nullptr, d_gT, d_uT, hsT,
+                              ldt, d_scores, workspace, workspace_bytes, A, H, I, E, dtype, stream);
 }
 
 int pk_grouped_swiglu_dgrad_dx(const void* d_g, const void* d_u, const void* w1, const void* w3,
@@ -1546,5 +2037,67 @@ int pk_grouped_swiglu_wgrad_scaled(const void* d_out, const void* hs, const void
   return wgrad_impl(d_out, 1, hs, d_g, d_u, x, row_map, row_map_div, starts, expert_order, d_w1, d_w2, d_w3,
                     accumulate, A, H, I, E, dtype, stream);
 }
+
+int pk_grouped_swiglu_wgrad_scaled_t(const void* d_out, const void* hsT, const void* d_gT, const void* d_uT,
+                                     int64_t ldt, const void* x, const int32_t* row_map, int64_t row_map_div,
+                                     const int32_t* starts, const int32_t* expert_order, void* d_w1,
+                                     void* d_w2, void* d_w3, int accumulate, int64_t A, int64_t H,
+                                     int64_t I, int64_t E, int dtype, pk_stream_t stream) {
+  int rc = check_common(A, H, I, E, dtype);
+  if (rc) return rc;
+  const int64_t need = pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype);
+  if (need <= 0) return PK_ERR_SHAPE;
+  // no routed rows: zero gradients (or nothing, when accumulating) from the kernel that needs no row map
+  if (A == 0) return wgrad_impl(nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, 1, starts, expert_order, d_w1, d_w2, d_w3,
+                                accumulate, A, H, I, E, dtype, stream);
+  if (!starts || !row_map || row_map_div <= 0 || row_map_div > 0x7fffffffll || ldt < need || ldt % 64 != 0) return PK_ERR_ARG;
+  if (d_w2 && (!d_out || !hsT)) return PK_ERR_ARG;
+  if (d_w1 && (!d_gT || !x)) return PK_ERR_ARG;
+  if (d_w3 && (!d_uT || !x)) return PK_ERR_ARG;
+  if (!all_aligned16({d_out, hsT, d_gT, d_uT, x, d_w1, d_w2, d_w3})) return PK_ERR_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  mf::WgradKcParams base = {};
+  base.ldt = ldt; base.ldr = H;
+  base.row_map = row_map; base.map_div = mf::make_fastdiv(row_map_div);
+  base.starts = starts; base.order = expert_order; base.E = (int32_t)E; base.total_rows = (int32_t)A;
+  base.accumulate = accumulate ? 1 : 0;
+  // skewed routing (experts of very different size) needs the dynamic hand-out of units; with a few
+  // hundred rows per expert the static one is a few per cent faster
+  const bool dynamic = A >= (int64_t)PK_WG_SHORTK_ROWS * E;
+  auto launch = [&](mf::WgradKcParams& p, bool a_kc) -> int {
+    const int64_t units = (int64_t)E * p.nprob * (p.M / 256) * (p.N / 256);
+    if (units > 0x7ffffff0ll) return PK_ERR_SHAPE;
+    const dim3 grid((unsigned)(units < mf::persistent_grid() ? mf::round_up_xcd(units) : mf::persistent_grid())), block(512);
+    if (dynamic) {
+      p.sched = mf::sched_slot_for_launch();
+      if (!p.sched) return PK_ERR_UNSUPPORTED;
+    }
+    const int id = a_kc ? pk_timing::K_SWIGLU_WGRAD_W13 : pk_timing::K_SWIGLU_WGRAD_W2;
+    if (a_kc && dynamic) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_kc_kernel<256, 256, 32, 2, 4, 4, true, true>), grid, block, 0, s, p);
+    else if (a_kc) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_kc_kernel<256, 256, 32, 2, 4, 4, true, false>), grid, block, 0, s, p);
+    else if (dynamic) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_kc_kernel<256, 256, 32, 4, 2, 4, false, true>), grid, block, 0, s, p);
+    else PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_kc_kernel<256, 256, 32, 4, 2, 4, false, false>), grid, block, 0, s, p);
+    PK_RETURN_IF_LAUNCH_FAILED();
+    return PK_OK;
+  };
+  if (d_w2) {   // d_w2[e][h][i] = sum_r d_out[token_r][h] * hs[r][i]: the transposed operand is the n side
+    mf::WgradKcParams p = base;
+    p.prob[0].T = (const bf16_t*)hsT; p.prob[0].R = (const bf16_t*)d_out; p.prob[0].C = (bf16_t*)d_w2;
+    p.nprob = 1; p.M = (int32_t)H; p.N = (int32_t)I;
+    rc = launch(p, false);
+    if (rc) return rc;
+  }
+  if (d_w1 || d_w3) {   // d_w1[e][i][h] = sum_r d_g[r][i] * x[token_r][h]: the transposed operand is the m side
+    mf::WgradKcParams p = base;
+    int n = 0;
+    if (d_w1) { p.prob[n].T = (const bf16_t*)d_gT; p.prob[n].R = (const bf16_t*)x; p.prob[n].C = (bf16_t*)d_w1; ++n; }
+    if (d_w3) { p.prob[n].T = (const bf16_t*)d_uT; p.prob[n].R = (const bf16_t*)x; p.prob[n].C = (bf16_t*)d_w3; ++n; }
+    p.nprob = n; p.M = (int32_t)I; p.N = (int32_t)H;
+    rc = launch(p, true);
+    if (rc) return rc;
+  }
+  return PK_OK;
+}
+
 
 }  // extern "C"

@@ -32,7 +32,7 @@ enum KernelId {
   K_SORT_SCATTER, K_COUNTS_TO_STARTS, K_PERMUTE_FWD, K_GATHER_REDUCE, K_COMBINE_BWD,
   K_SWIGLU_GATE_UP, K_SWIGLU_DOWN, K_SWIGLU_DGRAD_DH, K_SWIGLU_DGRAD_DX, K_SWIGLU_WGRAD,
   K_SIMT_GEMM, K_SWIGLU_ELEMENTWISE, K_BUCKET_PACK, K_BUCKET_UNPACK, K_BUCKET_ZERO, K_ADAMW,
-  K_RMSNORM_FWD, K_RMSNORM_BWD, K_MISC, K_COUNT
+  K_RMSNORM_FWD, K_RMSNORM_BWD, K_MISC, K_SWIGLU_WGRAD_W2, K_SWIGLU_WGRAD_W13, K_COUNT
 };
 // Brackets one kernel launch with two event records on `s` when timing is enabled
 // (pk_timing_enable); otherwise does nothing.

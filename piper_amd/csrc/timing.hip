@@ -28,7 +28,7 @@ const char* const kNames[K_COUNT] = {
     "sort_scatter", "counts_to_starts", "permute_fwd", "gather_reduce", "combine_bwd",
     "swiglu_gate_up", "swiglu_down", "swiglu_dgrad_dh", "swiglu_dgrad_dx", "swiglu_wgrad",
     "simt_gemm", "swiglu_elementwise", "bucket_pack", "bucket_unpack", "bucket_zero", "adamw",
-    "rmsnorm_fwd", "rmsnorm_bwd", "misc"};
+    "rmsnorm_fwd", "rmsnorm_bwd", "misc", "swiglu_wgrad_w2", "swiglu_wgrad_w13"};
 
 Scope::Scope(int id, hipStream_t s) : stream_(s), slot_(-1) {
   std::lock_guard<std::mutex> lk(g_mu);

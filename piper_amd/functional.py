@@ -126,25 +126,30 @@ class _BmmExpertsFn(torch.autograd.Function):
         return d_w1, d_w2, d_w3, d_x, None
 
 
-def _queue_expert_wgrad(params, d_y, h, d_g, d_u, x, starts, perm, top_k, order, scaled=False) -> None:
+def _queue_wgrad(params, wgrad) -> None:
+    """Queue `wgrad(**buffers)` -> (d_w1, d_w2, d_w3) for the weight pass; it accumulates into the
+    parameters' .grad, inside the kernel's epilogue when all three gradients exist already."""
     p1, p2, p3 = params
 
     def run():
         bufs = [_grad_target(p) for p in (p1, p2, p3)]
-        if all(acc for _, acc in bufs):     # accumulate in the kernel's epilogue
-            ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, p1.shape[0], row_map=perm, row_map_div=top_k,
-                                     expert_order=order, d_w1=bufs[0][0], d_w2=bufs[1][0], d_w3=bufs[2][0], accumulate=True,
-                                     scaled=scaled)
+        if all(acc for _, acc in bufs):
+            wgrad(d_w1=bufs[0][0], d_w2=bufs[1][0], d_w3=bufs[2][0], accumulate=True)
             return
-        g1, g2, g3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, p1.shape[0], row_map=perm,
-                                              row_map_div=top_k, expert_order=order, scaled=scaled)
-        for p, g in ((p1, g1), (p2, g2), (p3, g3)):
+        for p, g in zip((p1, p2, p3), wgrad()):
             if p.grad is None:
                 p.grad = g
             else:
                 p.grad += g
 
     _WGRAD_QUEUE.push(run)
+
+
+def _queue_expert_wgrad(params, d_y, h, d_g, d_u, x, starts, perm, top_k, order, scaled=False) -> None:
+    def wgrad(**kw):
+        return ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, params[0].shape[0], row_map=perm, row_map_div=top_k,
+                                        expert_order=order, scaled=scaled, **kw)
+    _queue_wgrad(params, wgrad)
 
 
 def _traced_without_data(*tensors) -> bool:
@@ -334,8 +339,24 @@ class _ExpertRegionFn(torch.autograd.Function):
         # combine backward folded into the d_h GEMM: d_out rows are gathered per routed row, the
         # score is applied in the epilogue; d_y below is d_out itself and h is score * h
         d_out = d_out.contiguous()
-        d_g, d_u, h, d_scores = ops.grouped_swiglu_dgrad_dh_scaled(d_out, perm, top_scores, w2, g, u, starts)
         d_y = d_out
+        # shapes with a K-contiguous weight-gradient path get d_g, d_u and score*h transposed as well
+        # (score*h only transposed): wgrad(...) below hides which of the two kernel pairs runs
+        if ops.transposed_ld(perm.numel(), x.shape[1], g.shape[1], E, g.dtype) > 0:
+            d_g, d_u, d_gT, d_uT, hsT, d_scores = ops.grouped_swiglu_dgrad_dh_scaled_t(d_out, perm, top_scores, w2, g, u, starts)
+            h = None
+
+            def wgrad(**kw):
+                return ops.grouped_swiglu_wgrad_scaled_t(d_out, hsT, d_gT, d_uT, x, starts, E, row_map=perm,
+                                                         row_map_div=top_k, expert_order=order, **kw)
+            wgrad_inputs = (d_out, hsT, d_gT, d_uT)
+        else:
+            d_g, d_u, h, d_scores = ops.grouped_swiglu_dgrad_dh_scaled(d_out, perm, top_scores, w2, g, u, starts)
+
+            def wgrad(**kw):
+                return ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k,
+                                                expert_order=order, scaled=True, **kw)
+            wgrad_inputs = (d_out, h, d_g, d_u)
         # The weight gradient (Piper's BWD_W) depends only on d_y, h, d_g, d_u and x; it runs on a
         # second stream next to the input gradient (BWD_I) so the two kernels fill each other's tails.
         d_w1 = d_w2 = d_w3 = None
@@ -345,7 +366,7 @@ class _ExpertRegionFn(torch.autograd.Function):
             # backward-input pass: the weight gradients of the experts and of the router gate are
             # queued with the tensors they need and computed by the weight pass
             p_gate, p_bias = ctx.params[0], ctx.params[1]
-            _queue_expert_wgrad(ctx.params[2:], d_y, h, d_g, d_u, x, starts, perm, top_k, order, scaled=True)
+            _queue_wgrad(ctx.params[2:], wgrad)
             d_xs = ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
             d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
             d_x32 = ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=need[0], d_w_gate=None, d_gate_bias=None)
@@ -379,9 +400,9 @@ class _ExpertRegionFn(torch.autograd.Function):
             if side is not None:
                 side.wait_stream(cur)
                 with torch.cuda.stream(side):
-                    d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k, expert_order=order, scaled=True)
+                    d_w1, d_w2, d_w3 = wgrad()
             else:
-                d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k, expert_order=order, scaled=True)
+                d_w1, d_w2, d_w3 = wgrad()
         d_xs = ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
         d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
         d_wg = torch.empty_like(w_gate) if need[1] else None
@@ -390,7 +411,7 @@ class _ExpertRegionFn(torch.autograd.Function):
         d_x = ops.permute_bwd(d_xs, inv_perm, top_k, addend_f32=d_x32) if need[0] else None
         if side is not None:
             cur.wait_stream(side)
-            for t in (d_y, h, d_g, d_u):     # allocated on the current stream, read on the side stream
+            for t in wgrad_inputs:           # allocated on the current stream, read on the side stream
                 t.record_stream(side)
             for t in (d_w1, d_w2, d_w3):     # allocated on the side stream, consumed on the current one
                 t.record_stream(cur)

@@ -285,6 +285,55 @@ def grouped_swiglu_dgrad_dh_scaled(d_out, perm, top_scores, w2, g, u, starts):
     return d_g, d_u, hs, d_scores
 
 
+def transposed_ld(A: int, H: int, I: int, E: int, dtype: torch.dtype) -> int:
+    """Row length of the transposed copies for the K-contiguous weight-gradient kernels, or 0 when
+    the shape / dtype has no such path."""
+    if dtype not in (torch.float32, torch.bfloat16):
+        return 0
+    return int(_lib.load().pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype_code(dtype)))
+
+
+def grouped_swiglu_dgrad_dh_scaled_t(d_out, perm, top_scores, w2, g, u, starts):
+    """grouped_swiglu_dgrad_dh_scaled with the outputs the weight gradient reads written transposed:
+    returns (d_g, d_u [A,I], d_gT, d_uT, hsT [I, ldt], d_scores [T,K] f32)."""
+    require_gpu(d_out)
+    E, H, I = w2.shape
+    A = perm.numel()
+    T, K = top_scores.shape
+    dev = d_out.device
+    ldt = transposed_ld(A, H, I, E, g.dtype)
+    _check(ldt > 0, "grouped_swiglu_dgrad_dh_scaled_t: shape without a transposed path")
+    d_g = torch.empty_like(g)
+    d_u = torch.empty_like(u)
+    d_gT, d_uT, hsT = (torch.empty((I, ldt), dtype=g.dtype, device=dev) for _ in range(3))
+    d_scores = torch.empty((T, K), dtype=torch.float32, device=dev)
+    ws_bytes = int(_lib.load().pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes(A, I))
+    ws = torch.empty(max(ws_bytes, 4) // 4, dtype=torch.float32, device=dev)
+    call("pk_grouped_swiglu_dgrad_dh_scaled_t", ptr(d_out.contiguous()), ptr(perm), K, ptr(top_scores.contiguous()),
+         ptr(w2.contiguous()), ptr(g), ptr(u), ptr(starts), ptr(d_g), ptr(d_u), ptr(d_gT), ptr(d_uT), ptr(hsT), ldt,
+         ptr(d_scores), ptr(ws), ws_bytes, A, H, I, E, dtype_code(g.dtype), current_stream(dev))
+    return d_g, d_u, d_gT, d_uT, hsT, d_scores
+
+
+def grouped_swiglu_wgrad_scaled_t(d_out, hsT, d_gT, d_uT, x, starts, E, *, row_map, row_map_div,
+                                  d_w1=None, d_w2=None, d_w3=None, accumulate=False, expert_order=None):
+    """Weight gradients from the transposed outputs of grouped_swiglu_dgrad_dh_scaled_t."""
+    require_gpu(d_out)
+    I, ldt = hsT.shape
+    H = d_out.shape[1]
+    A = row_map.numel()
+    dt, dev = d_out.dtype, d_out.device
+    if d_w1 is None:
+        d_w1 = torch.empty((E, I, H), dtype=dt, device=dev)
+        d_w2 = torch.empty((E, H, I), dtype=dt, device=dev)
+        d_w3 = torch.empty((E, I, H), dtype=dt, device=dev)
+        accumulate = False
+    call("pk_grouped_swiglu_wgrad_scaled_t", ptr(d_out.contiguous()), ptr(hsT), ptr(d_gT), ptr(d_uT), ldt, ptr(x.contiguous()),
+         ptr(row_map), row_map_div, ptr(starts), ptr(expert_order), ptr(d_w1), ptr(d_w2), ptr(d_w3), int(bool(accumulate)),
+         A, H, I, E, dtype_code(dt), current_stream(dev))
+    return d_w1, d_w2, d_w3
+
+
 def grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts):
     """Second half of the input gradient: d_x_sorted [A,H] = d_g . w1 + d_u . w3."""
     require_gpu(d_g)

@@ -122,6 +122,92 @@ def test_scaled_backward_matches_combine_bwd_then_dgrad(dev, dtype, counts, H, I
             assert float(dw2[e].abs().max()) == 0.0
 
 
+T_CASES = [
+    # ragged around the 8-row padding and the 32-row k-tile, empty experts, one long expert
+    ([0, 1, 7, 8, 9, 31, 32, 33, 0, 300, 64, 255], 256, 256),
+    ([700, 0, 0, 2], 512, 256),
+    ([256] * 6, 256, 512),
+]
+
+
+@pytest.mark.parametrize("counts,H,I", T_CASES)
+def test_transposed_backward_pair_matches_the_plain_pair(dev, counts, H, I):
+    """pk_grouped_swiglu_dgrad_dh_scaled_t / pk_grouped_swiglu_wgrad_scaled_t (one operand of every
+    weight-gradient GEMM K-contiguous, persistent workgroups) against
+    pk_grouped_swiglu_dgrad_dh_scaled / pk_grouped_swiglu_wgrad_scaled on the same inputs, against
+    fp32 autograd through the oracle, and the layout of the transposed copies."""
+    print(f"[case] transposed backward counts={counts} H={H} I={I}", flush=True)
+    K = 2
+    A = int(sum(counts))
+    if A % K:
+        counts = list(counts); counts[-1] += 1; A += 1
+    T, E = A // K, len(counts)
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(21)
+    _, w1, w2, w3, _, cnt = _make(6, counts, H, I, dtype)
+    perm = torch.randperm(A, generator=gen).to(torch.int32)
+    tok = perm.long() // K
+    x_tok = torch.randn(T, H, generator=gen).to(dtype)
+    scores = torch.rand(T, K, generator=gen) + 0.1
+    d_out = torch.randn(T, H, generator=gen).to(dtype)
+    XT, W1, W2, W3, PERM, SC, DO = (t.to(dev) for t in (x_tok, w1, w2, w3, perm, scores, d_out))
+    starts = ops.counts_to_starts(cnt.to(dev))
+    ldt = ops.transposed_ld(A, H, I, E, dtype)
+    assert ldt >= ((A + 63) // 64 + E) * 64 and ldt % 256 == 128
+    assert ops.transposed_ld(A, H + 128, I, E, dtype) == 0 and ops.transposed_ld(A, H, I, E, torch.float32) == 0
+    _, g, u, _ = ops.grouped_swiglu_fwd(XT, W1, W2, W3, starts, row_map=PERM, row_map_div=K)
+
+    d_g, d_u, hs, d_s = ops.grouped_swiglu_dgrad_dh_scaled(DO, PERM, SC, W2, g, u, starts)
+    # poison what the transposed call allocates next, so untouched pad columns would show as NaN
+    junk = torch.full((3 * I * ldt + 16,), float("nan"), dtype=dtype, device=dev)
+    del junk
+    d_g2, d_u2, d_gT, d_uT, hsT, d_s2 = ops.grouped_swiglu_dgrad_dh_scaled_t(DO, PERM, SC, W2, g, u, starts)
+    assert torch.equal(d_g, d_g2) and torch.equal(d_u, d_u2) and torch.equal(d_s, d_s2)
+    st = starts.cpu().tolist()
+    for e, c in enumerate(counts):
+        p0 = (st[e] // 64) * 64 + 64 * e
+        c8 = (c + 7) // 8 * 8
+        for full, tr in ((d_g, d_gT), (d_u, d_uT), (hs, hsT)):
+            blk = tr[:, p0:p0 + c8]
+            assert torch.equal(blk[:, :c], full[st[e]:st[e] + c].t()), f"expert {e}"
+            assert torch.count_nonzero(blk[:, c:]).item() == 0, f"pad columns of expert {e}"
+
+    ref = ops.grouped_swiglu_wgrad(DO, hs, d_g, d_u, XT, starts, E, row_map=PERM, row_map_div=K, scaled=True)
+    order = torch.argsort(cnt, descending=True, stable=True).to(torch.int32).to(dev)
+    for eo in (None, order):
+        got = ops.grouped_swiglu_wgrad_scaled_t(DO, hsT, d_gT, d_uT, XT, starts, E, row_map=PERM, row_map_div=K, expert_order=eo)
+        for a, b, name in zip(got, ref, ("d_w1", "d_w2", "d_w3")):
+            # same products, same fp32 summation order over the rows: equal up to the last bf16 bit
+            assert rel_err(a, b) <= 2.0 ** -7, name
+            for e, c in enumerate(counts):
+                if c == 0:
+                    assert float(a[e].abs().max()) == 0.0
+    # fp32 reference through the oracle
+    x_sorted = x_tok[tok]
+    xr, w1r, w2r, w3r = (t.float().requires_grad_(True) for t in (x_sorted, w1, w2, w3))
+    y_ref = O.grouped_swiglu(w1r, w2r, w3r, xr, cnt)
+    out_ref = torch.zeros(T, H).index_add(0, tok, y_ref * scores.reshape(-1)[perm.long()].unsqueeze(1))
+    dw_ref = torch.autograd.grad(out_ref, (w1r, w2r, w3r), d_out.float())
+    for a, b in zip(got, (dw_ref[0], dw_ref[1], dw_ref[2])):
+        assert rel_err(a, b) <= BF16_TOL
+    # accumulate: adds to what is there, twice gives 2x (+ one rounding)
+    acc = [t.clone() for t in got]
+    ops.grouped_swiglu_wgrad_scaled_t(DO, hsT, d_gT, d_uT, XT, starts, E, row_map=PERM, row_map_div=K,
+                                      d_w1=acc[0], d_w2=acc[1], d_w3=acc[2], accumulate=True, expert_order=order)
+    for a, b in zip(acc, got):
+        assert rel_err(a, 2 * b.float()) <= 2.0 ** -7
+    # argument checks: a row length below the query's, and a shape without the path
+    with pytest.raises(RuntimeError):
+        _lib_call_short_ld(DO, hsT, d_gT, d_uT, XT, PERM, starts, E, H, I, A, K, ldt - 64)
+
+
+def _lib_call_short_ld(DO, hsT, d_gT, d_uT, XT, PERM, starts, E, H, I, A, K, ldt):
+    from piper_amd._lib import call, current_stream, dtype_code, ptr
+    w = torch.empty((E, I, H), dtype=DO.dtype, device=DO.device)
+    call("pk_grouped_swiglu_wgrad_scaled_t", ptr(DO), ptr(hsT), ptr(d_gT), ptr(d_uT), ldt, ptr(XT), ptr(PERM), K, ptr(starts),
+         ptr(None), ptr(w), ptr(None), ptr(None), 0, A, H, I, E, dtype_code(DO.dtype), current_stream(DO.device))
+
+
 def test_mfma_path_agrees_with_fma_path(dev):
     """bf16 shapes outside the MFMA tiling (H or I not a multiple of 128) run on the FMA kernel."""
     print("[case] bf16 fallback shapes", flush=True)

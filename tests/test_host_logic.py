@@ -98,3 +98,20 @@ def test_kernels_refuse_cpu_tensors():
         ops.route_topk(torch.zeros(4, 8), 2, True)
     with pytest.raises(RuntimeError, match="GPU only"):
         ops.bucket_zero(torch.zeros(16))
+
+
+def test_annotate_is_traceable_by_dynamo_fullgraph():
+    """The model's forward runs under Dynamo with fullgraph=True (src/compile.py:273): the scope
+    bookkeeping must not break the graph."""
+    import torch
+
+    def fn(x):
+        with annotate("PP"):
+            with annotate("EP"):
+                y = x + 1
+        return y * 2
+
+    reset_annotation_state()
+    out = torch.compile(fn, fullgraph=True, backend="eager")(torch.ones(3))
+    assert torch.equal(out, torch.full((3,), 4.0))
+    assert current_annotations() == ()
