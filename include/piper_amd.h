@@ -104,6 +104,19 @@ PK_API int pk_sort_by_expert(const int32_t* top_idx, int64_t A, int64_t E, int32
                       int32_t* starts, int32_t* perm, int32_t* inv_perm, int32_t* order,
                       void* workspace, int64_t workspace_bytes, pk_stream_t stream);
 
+/* pk_sort_by_expert for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * inputs, outputs and result as pk_sort_by_expert; the per-chunk histograms live in a fixed array
+ * inside the library (PK_SORT_STATIC_WORDS int32 per GPU, held until the process ends) instead of a
+ * caller workspace, and nothing is allocated.  Limit: ceil(A / 512) * E <= PK_SORT_STATIC_WORDS,
+ * otherwise PK_ERR_WORKSPACE and nothing is launched.  All calls on one GPU share the array: calls
+ * that overlap on one GPU (different streams or threads) race; calls on one stream are ordered.
+ * The array needs no clearing between calls (every word a call reads it has written before). */
+#define PK_SORT_STATIC_WORDS (256 * 1024)
+PK_API int pk_sort_by_expert_static(const int32_t* top_idx, int64_t A, int64_t E, int32_t* counts,
+                             int32_t* starts, int32_t* perm, int32_t* inv_perm, int32_t* order,
+                             pk_stream_t stream);
+
 /* starts[E+1] (i32) from counts[E] given as int32 (counts_is_i64 == 0) or int64.
  * For callers that hand pk_grouped_swiglu_* a `num_tokens_per_expert` tensor
  * (qwen3_bmm_experts_patch.py:24-27). */

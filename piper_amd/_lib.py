@@ -34,6 +34,7 @@ SIGNATURES = {
     "pk_gate_logits_bwd": (_c_int, [_p, _p, _c_int, _p, _p, _p, _p, _c_int, _c_i64, _c_i64, _c_i64, _p, _c_i64, _p]),
     "pk_sort_workspace_bytes": (_c_i64, [_c_i64, _c_i64]),
     "pk_sort_by_expert": (_c_int, [_p, _c_i64, _c_i64, _p, _p, _p, _p, _p, _p, _c_i64, _p]),
+    "pk_sort_by_expert_static": (_c_int, [_p, _c_i64, _c_i64, _p, _p, _p, _p, _p, _p]),
     "pk_counts_to_starts": (_c_int, [_p, _c_int, _c_i64, _p, _p]),
     "pk_permute_fwd": (_c_int, [_p, _c_int, _p, _p, _c_i64, _c_i64, _c_i64, _p]),
     "pk_permute_bwd": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p]),

@@ -1,6 +1,7 @@
 // Routing: gate logits, wavefront softmax/top-k (+ backward), stable counting sort by expert.
 #include "pk_common.h"
 #include "mfma_x3_gemm.h"
+#include <mutex>
 
 namespace {
 
@@ -307,6 +308,27 @@ __global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ d
   if (threadIdx.x == 0) d_bias[e] = accumulate ? d_bias[e] + s : s;
 }
 
+// Scratch of pk_sort_by_expert_static: the per-chunk histograms of the counting sort.  Every GPU
+// the library runs on holds its own copy of the array (PK_SORT_STATIC_WORDS * 4 bytes) until the
+// process ends.  In host code the name `scratch` is only a handle for hipGetSymbolAddress: the
+// address a kernel can use is looked up once per device, with that device current, and kept.
+static __device__ __align__(256) int32_t scratch[PK_SORT_STATIC_WORDS];
+
+int32_t* sort_scratch_for_current_device() {
+  constexpr int MAX_DEV = 64;
+  static int32_t* ptr[MAX_DEV] = {};
+  static std::mutex mu;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+    ptr[dev] = static_cast<int32_t*>(p);
+  }
+  return ptr[dev];
+}
+
 }  // namespace
 
 extern "C" {
@@ -505,6 +527,19 @@ int pk_sort_by_expert(const int32_t* top_idx, int64_t A, int64_t E, int32_t* cou
     PK_RETURN_IF_LAUNCH_FAILED();
   }
   return PK_OK;
+}
+
+int pk_sort_by_expert_static(const int32_t* top_idx, int64_t A, int64_t E, int32_t* counts,
+                             int32_t* starts, int32_t* perm, int32_t* inv_perm, int32_t* order,
+                             pk_stream_t stream) {
+  if (A < 0 || E <= 0) return PK_ERR_ARG;
+  if (E > PK_MAX_EXPERTS || A > 0x7fffffffll) return PK_ERR_SHAPE;
+  // the per-chunk histograms must fit the fixed scratch array
+  const int64_t need = pk_sort_workspace_bytes(A, E);
+  if (need > (int64_t)sizeof(int32_t) * PK_SORT_STATIC_WORDS) return PK_ERR_WORKSPACE;
+  int32_t* ws = sort_scratch_for_current_device();
+  if (!ws) return PK_ERR_UNSUPPORTED;
+  return pk_sort_by_expert(top_idx, A, E, counts, starts, perm, inv_perm, order, ws, need, stream);
 }
 
 int pk_counts_to_starts(const void* counts, int counts_is_i64, int64_t E, int32_t* starts,
