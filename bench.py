@@ -33,6 +33,7 @@ def parse_args():
     ap.add_argument("--workload", choices=["cfg3", "cfg4"], default="cfg3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bucket", action="store_true")
+    ap.add_argument("--no-cfg4", action="store_true", help="skip the cfg4 sub-object of the default run")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB fp32 device copy (pack_kernel<float,float>) so that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled to a known size")
@@ -47,13 +48,18 @@ def kernel_flops(cfg) -> dict:
         "swiglu_down": one,
         "swiglu_dgrad_dh": one,
         "swiglu_dgrad_dx": 2 * one,  # d_g.w1 + d_u.w3
-        "swiglu_wgrad": 3 * one,     # d_w1, d_w2, d_w3 in one launch
+        "swiglu_wgrad": 3 * one,     # d_w1, d_w2, d_w3 in one launch (shapes without the K-contiguous path)
+        "swiglu_wgrad_w2": one,      # d_w2 = d_out^T (score h)
+        "swiglu_wgrad_w13": 2 * one,  # d_w1 = d_g^T x and d_w3 = d_u^T x in one launch
     }
 
 
 def kernel_bytes(cfg) -> dict:
     """Algorithmic HBM bytes of ONE launch of each GEMM kernel: every operand read once, every
-    result written once (bf16).  A = routed rows, T = tokens, E experts, H hidden, I intermediate."""
+    result written once (bf16).  A = routed rows, T = tokens, E experts, H hidden, I intermediate.
+    The transposed copies that the scaled SwiGLU backward writes for the weight gradient are an
+    implementation choice, not algorithmic work: they count as one write / one read of d_g, d_u
+    and score*h like the row-major tensors they stand in for."""
     A, T, E, H, I = cfg.routed_rows, cfg.tokens, cfg.num_experts, cfg.hidden, cfg.inter
     w = 2.0 * E * I * H          # one expert weight tensor
     return {
@@ -63,16 +69,16 @@ def kernel_bytes(cfg) -> dict:
         "swiglu_dgrad_dh": w + 2.0 * T * H + 2 * 2.0 * A * I + 3 * 2.0 * A * I + 4.0 * A * (I / 64),
         "swiglu_dgrad_dx": 2 * w + 2 * 2.0 * A * I + 2.0 * A * H,       # w1,w3 + d_g,d_u -> d_x rows
         "swiglu_wgrad": 2 * 2.0 * T * H + 3 * 2.0 * A * I + 3 * w,      # d_out,x (each token once), score*h,d_g,d_u -> d_w1..3
+        "swiglu_wgrad_w2": 2.0 * T * H + 2.0 * A * I + w,               # d_out (each token once), score*h -> d_w2
+        "swiglu_wgrad_w13": 2.0 * T * H + 2 * 2.0 * A * I + 2 * w,      # x (each token once), d_g, d_u -> d_w1, d_w3
     }
 
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the cfg3 workload,
-# scaled by what the same counters read for a plain device copy of known size
-# (profiles/bench_cfg3_hbm_traffic.md).  None where no measurement is committed.
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
+# counters read for a plain device copy of known size.  The numbers and the commands that produced
+# them are in the file named here; a kernel without a committed measurement reports null.
+TRAFFIC_SOURCE = "profiles/bench_hbm_traffic.md"
 MEASURED_TRAFFIC_BYTES = {
-    "cfg3-qwen3-30b-a3b": {
-        "swiglu_wgrad": (409 + 1197) * 1e6,
-    },
 }
 
 
@@ -170,13 +176,18 @@ def bench_bucket(steps: int, warmup: int):
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    _lib.timing_enable(True)
-    _lib.timing_collect()
+    # timed region: nothing but the two launches per step on the stream
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    # per-kernel durations: a second pass with each launch bracketed by HIP events
+    _lib.timing_enable(True)
+    _lib.timing_collect()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
     records = _lib.timing_collect()
     _lib.timing_enable(False)
     n_elems = sum(numels)
@@ -186,16 +197,21 @@ def bench_bucket(steps: int, warmup: int):
     pack_bytes = 6.0 * n_elems            # read bf16 grad, write fp32 bucket
     adam_bytes = 30.0 * total             # read g,p,m,v (16) + write p,m,v (12) + bf16 parameter (2)
     agg_gbs = (pack_bytes + adam_bytes) * steps / elapsed / 1e9
+    traffic = MEASURED_TRAFFIC_BYTES.get("cfg2", {}).get("pack+adamw")
     return {
         "metric": "bucket pack + fused AdamW HBM GB/s",
         "value": agg_gbs, "unit": "GB/s", "ms_per_step": elapsed / steps * 1e3,
         "config": {"workload": "cfg2: 96 tensors of two Qwen3-30B-A3B layers, bf16 grads / fp32 master",
                    "tensors": len(shapes), "elements": n_elems, "bucket_elements": total},
         "bytes_per_element": {"pack": 6, "adamw": 30},
+        "per_kernel_source": "second pass with each launch bracketed by HIP events; value and ms_per_step are from the "
+                             "timed region without brackets",
         "pack": {"avg_ms": pack_avg, "GB/s": pack_bytes / pack_avg / 1e6, "frac": pack_bytes / pack_avg / 1e6 / HBM_PEAK_GBS},
         "adamw": {"avg_ms": adam_avg, "GB/s": adam_bytes / adam_avg / 1e6, "frac": adam_bytes / adam_avg / 1e6 / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "achieved": agg_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": agg_gbs / HBM_PEAK_GBS, "traffic": None},
+                     "frac": agg_gbs / HBM_PEAK_GBS, "traffic": traffic,
+                     "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
+                     "bytes_per_step": pack_bytes + adam_bytes},
     }
 
 
@@ -233,6 +249,63 @@ def cpu_baseline(cfg):
                       f"fwd+bwd, best of 2 after 1 warm-up ({t:.2f} s per pass)"}
 
 
+def region_result(cfg, steps: int, warmup: int) -> dict:
+    """Tokens/s, fraction of the bf16 MFMA peak and the roofline of the dominant GEMM kernel for one
+    expert-region configuration."""
+    elapsed, kernels = bench_region(cfg, steps, warmup)
+    host_enqueue = kernels.pop("__host_enqueue_s")
+    dominant = kernels.pop("__dominant")
+    ms_per_step = elapsed / steps * 1e3
+    tokens_per_s = cfg.tokens * steps / elapsed
+    gemm_flops_step = cfg.gemm_flops_per_token * cfg.tokens
+    mfma_frac_region = gemm_flops_step / (ms_per_step * 1e-3) / (MFMA_BF16_PEAK_TFLOPS * 1e12)
+
+    flops = kernel_flops(cfg)
+    gemm_kernels = {k: v for k, v in kernels.items() if k in flops}
+    dom = gemm_kernels[dominant]
+    nbytes = kernel_bytes(cfg)
+    # the roofline that bounds the kernel: below the ridge point (peak flops / peak bandwidth) of
+    # the published peaks, moving its algorithmic bytes takes longer than its algorithmic flops
+    intensity = flops[dominant] / nbytes[dominant]
+    ridge = MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+    traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name, {}).get(dominant)
+    if intensity < ridge:
+        achieved = nbytes[dominant] / (dom["avg_ms"] * 1e-3) / 1e9
+        roof = {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBS, "traffic": traffic}
+    else:
+        achieved = flops[dominant] / (dom["avg_ms"] * 1e-3) / 1e12
+        roof = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic}
+    roof.update({"traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
+                 "flops_per_launch": flops[dominant], "bytes_per_launch": nbytes[dominant],
+                 "flops_per_byte": intensity, "avg_launch_ms": dom["avg_ms"],
+                 "tflops": flops[dominant] / (dom["avg_ms"] * 1e-3) / 1e12})
+    return {
+        "metric": "expert-region fwd+bwd tokens/s",
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": ms_per_step,
+        "dtype": "bf16",
+        "config": {"workload": f"{cfg.name}: T={cfg.tokens} H={cfg.hidden} E={cfg.num_experts} top{cfg.top_k} "
+                               f"I={cfg.inter}, bf16 experts, fp32 router, fwd+bwd incl. router and all expert weight grads",
+                   "tokens_per_step": cfg.tokens},
+        "host_enqueue_ms_per_step": host_enqueue / steps * 1e3,
+        "mfma_frac_of_peak_region": mfma_frac_region,
+        "gemm_tflops_region": gemm_flops_step / (ms_per_step * 1e-3) / 1e12,
+        "roofline": roof,
+        # per-kernel table: from a separate, untimed pass with EVERY launch bracketed by HIP events, which
+        # costs the stream about 5 % (so the entries add up to more than ms_per_step); only the dominant
+        # kernel's entry and the roofline's launch time come from the timed region itself
+        "kernels_ms_per_step": {k: round(v["ms_per_step"], 4) for k, v in sorted(kernels.items(), key=lambda kv: -kv[1]["ms_per_step"])},
+        "kernels_ms_per_step_source": "untimed pass with every launch bracketed by HIP events (about 5 % slower than "
+                                      "the timed region); the dominant kernel's entry is from the timed region",
+        "gemm_kernels_tflops": {k: round(flops[k] / (v["avg_ms"] * 1e-3) / 1e12, 1) for k, v in gemm_kernels.items()},
+    }
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -257,57 +330,13 @@ def main():
             ops.bucket_pack([src], [0], dst, accumulate=False)   # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
-    elapsed, kernels = bench_region(cfg, args.steps, args.warmup)
-    host_enqueue = kernels.pop("__host_enqueue_s")
-    dominant = kernels.pop("__dominant")
-    ms_per_step = elapsed / args.steps * 1e3
-    tokens_per_s = cfg.tokens * args.steps / elapsed
-    gemm_flops_step = cfg.gemm_flops_per_token * cfg.tokens
-    mfma_frac_region = gemm_flops_step / (ms_per_step * 1e-3) / (MFMA_BF16_PEAK_TFLOPS * 1e12)
-
-    flops = kernel_flops(cfg)
-    gemm_kernels = {k: v for k, v in kernels.items() if k in flops}
-    dom = gemm_kernels[dominant]
-    nbytes = kernel_bytes(cfg)
-    # the roofline that bounds the kernel: below the ridge point (peak flops / peak bandwidth) of
-    # the published peaks, moving its algorithmic bytes takes longer than its algorithmic flops
-    intensity = flops[dominant] / nbytes[dominant]
-    ridge = MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
-    traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name, {}).get(dominant)
-    if intensity < ridge:
-        achieved = nbytes[dominant] / (dom["avg_ms"] * 1e-3) / 1e9
-        roof = {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS, "traffic": traffic}
-    else:
-        achieved = flops[dominant] / (dom["avg_ms"] * 1e-3) / 1e12
-        roof = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
-                "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic}
-    roof.update({"flops_per_launch": flops[dominant], "bytes_per_launch": nbytes[dominant],
-                 "flops_per_byte": intensity, "avg_launch_ms": dom["avg_ms"],
-                 "tflops": flops[dominant] / (dom["avg_ms"] * 1e-3) / 1e12})
-    result = {
-        "metric": "expert-region fwd+bwd tokens/s",
-        "value": tokens_per_s,
-        "unit": "tokens/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
-        "config": {"workload": f"{cfg.name}: T={cfg.tokens} H={cfg.hidden} E={cfg.num_experts} top{cfg.top_k} "
-                               f"I={cfg.inter}, bf16 experts, fp32 router, fwd+bwd incl. router and all expert weight grads",
-                   "tokens_per_step": cfg.tokens},
-        "host_enqueue_ms_per_step": host_enqueue / args.steps * 1e3,
-        "mfma_frac_of_peak_region": mfma_frac_region,
-        "gemm_tflops_region": gemm_flops_step / (ms_per_step * 1e-3) / 1e12,
-        "roofline": roof,
-        "kernels_ms_per_step": {k: round(v["ms_per_step"], 4) for k, v in sorted(kernels.items(), key=lambda kv: -kv[1]["ms_per_step"])},
-        "gemm_kernels_tflops": {k: round(flops[k] / (v["avg_ms"] * 1e-3) / 1e12, 1) for k, v in gemm_kernels.items()},
-    }
+    result = region_result(cfg, args.steps, args.warmup)
+    result.update({"n_gpus": 1, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "data": "synthetic"})
+    if args.workload == "cfg3" and not args.no_cfg4:
+        # the compute-bound configuration (16384 tokens, Zipf-skewed routing) in the same run
+        c4 = region_result(CFG4, args.steps, args.warmup)
+        result["cfg4"] = {k: c4[k] for k in ("value", "unit", "ms_per_step", "config", "mfma_frac_of_peak_region",
+                                             "gemm_tflops_region", "roofline", "kernels_ms_per_step", "gemm_kernels_tflops")}
     if not args.no_bucket:
         result["bucket"] = bench_bucket(max(5, args.steps), max(2, args.warmup))
     if not args.no_cpu_baseline:
