@@ -36,7 +36,7 @@ def gate_logits(x: torch.Tensor, w_gate: torch.Tensor, gate_bias: torch.Tensor |
     return logits
 
 
-def route_topk(logits: torch.Tensor, top_k: int, route_norm: bool, route_scale: float = 1.0):
+def route_topk(logits: torch.Tensor, top_k: int, route_norm: bool, route_scale: float = 1.0, top_idx=None):
     """softmax over experts (fp32), top-k with ties to the LOWER expert index, optional
     renormalisation of the selected scores (MoEArgs score_func="softmax", route_norm,
     route_scale: qwen3.py:41-44,170-173).
@@ -47,8 +47,13 @@ def route_topk(logits: torch.Tensor, top_k: int, route_norm: bool, route_scale: 
     [2, 3]); a stable descending sort returns equal keys in ascending index order."""
     logits = logits.float()
     scores = torch.softmax(logits, dim=-1)
-    order = torch.sort(logits, dim=-1, descending=True, stable=True).indices
-    top_idx = order[:, :top_k].contiguous()
+    if top_idx is None:
+        order = torch.sort(logits, dim=-1, descending=True, stable=True).indices
+        top_idx = order[:, :top_k].contiguous()
+    else:
+        # a selection made elsewhere (a test hands over the device's indices so that a token on a
+        # near-tie, which bf16 activations can tip either way, is routed alike on both sides)
+        top_idx = top_idx.long()
     top_scores = scores.gather(1, top_idx)
     if route_norm:
         top_scores = top_scores / (top_scores.sum(dim=-1, keepdim=True) + 1e-20)
@@ -134,12 +139,12 @@ def unpermute_combine(y_sorted: torch.Tensor, perm: torch.Tensor, top_scores: to
     return out.to(out_dtype or y_sorted.dtype)
 
 
-def moe_forward(x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale=1.0, compute_dtype=None):
+def moe_forward(x, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale=1.0, compute_dtype=None, top_idx=None):
     """AnnotatedMoE.forward on x [T,H] (qwen3.py:233-289).  Returns (out, aux) where aux holds the
     routing tables.  Differentiable w.r.t. x, w_gate, gate_bias, w1, w2, w3."""
     E = w1.shape[0]
     logits = gate_logits(x, w_gate, gate_bias)
-    top_scores, top_idx = route_topk(logits, top_k, route_norm, route_scale)
+    top_scores, top_idx = route_topk(logits, top_k, route_norm, route_scale, top_idx=top_idx)
     counts, starts, perm, inv_perm = sort_by_expert(top_idx, E)
     routed = permute(x, perm, top_k)
     y = grouped_swiglu(w1, w2, w3, routed, counts, compute_dtype=compute_dtype)
@@ -158,8 +163,8 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.T
 
 
 def moe_block(h, norm_weight, w_gate, gate_bias, w1, w2, w3, top_k, route_norm, route_scale=1.0, norm_eps=1e-6,
-              compute_dtype=None):
+              compute_dtype=None, top_idx=None):
     """h + moe(ffn_norm(h)) (qwen3.py:313-314) on h [T,H]."""
     out, aux = moe_forward(rmsnorm(h, norm_weight, norm_eps), w_gate, gate_bias, w1, w2, w3, top_k, route_norm,
-                           route_scale, compute_dtype=compute_dtype)
+                           route_scale, compute_dtype=compute_dtype, top_idx=top_idx)
     return h + out, aux

@@ -53,6 +53,42 @@ def _gpu_fwd_bwd(inp, cfg, dev, fused=True):
     return out.detach(), g
 
 
+def _torch_fp32_region_on_device(d, cfg, top_idx):
+    """The region in fp32 with torch's own operators on the GPU (softmax, gather, per-expert
+    matmuls, index_add), forward and autograd backward, routed with the given expert indices.
+    d: the inputs on the device.  Returns (out, gradients by name)."""
+    K, E, T = cfg.top_k, cfg.num_experts, cfg.tokens
+    names = ("x", "w_gate", "w1", "w2", "w3")
+    leaf = {k: d[k].detach().float().requires_grad_(True) for k in names}
+    bias = d["gate_bias"].detach().float().requires_grad_(True) if d["gate_bias"] is not None else None
+    logits = leaf["x"] @ leaf["w_gate"].t()
+    if bias is not None:
+        logits = logits + bias
+    ts = torch.softmax(logits, dim=-1).gather(1, top_idx.long())
+    if cfg.route_norm:
+        ts = ts / (ts.sum(dim=-1, keepdim=True) + 1e-20)
+    ts = ts * cfg.route_scale
+    flat = top_idx.reshape(-1).long()
+    perm = torch.argsort(flat, stable=True)
+    counts = torch.bincount(flat, minlength=E).cpu().tolist()
+    tok = perm // K
+    routed = leaf["x"][tok]
+    outs, start = [], 0
+    for e in range(E):
+        xe = routed[start:start + counts[e]]
+        h = torch.nn.functional.silu(xe @ leaf["w1"][e].t()) * (xe @ leaf["w3"][e].t())
+        outs.append(h @ leaf["w2"][e].t())
+        start += counts[e]
+    y = torch.cat(outs, 0)
+    out = torch.zeros(T, cfg.hidden, device=y.device).index_add(0, tok, y * ts.reshape(-1)[perm].unsqueeze(1))
+    targets = [leaf[k] for k in names] + ([bias] if bias is not None else [])
+    grads = torch.autograd.grad(out, targets, d["d_out"].float())
+    g = dict(zip(names, grads))
+    if bias is not None:
+        g["gate_bias"] = grads[-1]
+    return out.detach(), g
+
+
 def test_config1_exact_four_microbatches_then_bucket_adamw(dev):
     """Config 1 as specified: fp32, 4 microbatches x 256 tokens, fwd+bwd, all grads flattened into
     one bucket, one AdamW step."""
@@ -275,8 +311,27 @@ def test_full_size_properties(dev, cfg):
         assert rel_err(y[s0:s1], ye) <= BF16_TOL
         assert rel_err(dx[s0:s1], gx) <= BF16_TOL
         assert rel_err(dw1[e], g1) <= BF16_TOL and rel_err(dw2[e], g2) <= BF16_TOL and rel_err(dw3[e], g3) <= BF16_TOL
-    # whole region: linear in the upstream gradient (scale by 2 -> every gradient doubles)
+    # The fused region (the path bench.py times: gather fused into the GEMM loads, combine backward
+    # folded into the d_h GEMM, transposed copies, persistent weight-gradient kernels) against an
+    # fp32 evaluation of the whole region with library matmuls on the same device, routed with the
+    # same indices (bit-exact against the CPU oracle given the logits, see above): every output and
+    # every gradient, all experts, plus the least / median / most loaded expert each on its own scale.
     out1, g1_ = _gpu_fwd_bwd(inp, cfg, dev)
+    out_ref, g_ref = _torch_fp32_region_on_device(d, cfg, idx)
+    assert rel_err(out1, out_ref) <= BF16_TOL
+    for k in g1_:
+        assert rel_err(g1_[k], g_ref[k]) <= BF16_TOL, f"{k}: {rel_err(g1_[k], g_ref[k]):.4f}"
+    for e in (int(order[0]), int(order[E // 2]), int(order[-1])):
+        for k in ("w1", "w2", "w3"):
+            if int(c_ref[e]) == 0:
+                assert float(g1_[k][e].abs().max()) == 0.0
+            else:
+                assert rel_err(g1_[k][e], g_ref[k][e]) <= BF16_TOL, (k, e, int(c_ref[e]))
+        rows = (perm[int(st_ref[e]):int(st_ref[e + 1])].long() // K)
+        if rows.numel():
+            assert rel_err(g1_["x"][rows], g_ref["x"][rows]) <= BF16_TOL
+    del out_ref, g_ref
+    # whole region: linear in the upstream gradient (scale by 2 -> every gradient doubles)
     inp2 = dict(inp)
     inp2["d_out"] = inp["d_out"] * 2
     out2, g2_ = _gpu_fwd_bwd(inp2, cfg, dev)

@@ -143,27 +143,34 @@ def test_gate_logits_backward(dev, dtype):
     assert rel_err(dw, 2 * dw_ref) <= F32_TOL and rel_err(db, 2 * db_ref) <= F32_TOL
 
 
-def test_end_to_end_routing_from_activations(dev):
-    """x, W -> indices.  The GPU gate sums in a different order than the CPU, so logits differ in
-    the last bits; every index that differs from the oracle must sit on a near-tie (margin below
-    1e-4), and given the GPU's own logits the selection is bit-exact."""
-    _note("routing end to end (cfg3 shape)")
-    from piper_amd.configs import CFG3, make_expert_region_inputs
-    inp = make_expert_region_inputs(CFG3)
-    x, w = inp["x"], inp["w_gate"]
-    logits_gpu = ops.gate_logits(x.to(dev), w.to(dev)).cpu()
-    logits_ref = O.gate_logits(x, w)
+@pytest.mark.parametrize("name", ["cfg3", "cfg4"])
+def test_end_to_end_routing_from_activations(dev, name):
+    """x, W (, bias) -> indices at the full size of both expert-region configurations.  The GPU gate
+    sums in a different order than the CPU, so logits differ in the last bits; every token whose
+    indices differ from the oracle's must sit on a near-tie (margin below 1e-4 between two of its
+    nine largest logits), their number is printed and bounded, and given the GPU's own logits the
+    selection is bit-exact."""
+    from piper_amd.configs import CFG3, CFG4, make_expert_region_inputs
+    cfg = CFG3 if name == "cfg3" else CFG4
+    _note(f"routing end to end ({name} shape)")
+    inp = make_expert_region_inputs(cfg)
+    x, w, b = inp["x"], inp["w_gate"], inp["gate_bias"]
+    logits_gpu = ops.gate_logits(x.to(dev), w.to(dev), None if b is None else b.to(dev)).cpu()
+    logits_ref = O.gate_logits(x, w, b)
     assert rel_err(logits_gpu, logits_ref) <= F32_TOL
-    _, i_gpu = ops.route_topk(logits_gpu.to(dev), 8, True)
-    _, i_from_gpu_logits = O.route_topk(logits_gpu, 8, True)
+    K = cfg.top_k
+    _, i_gpu = ops.route_topk(logits_gpu.to(dev), K, True)
+    _, i_from_gpu_logits = O.route_topk(logits_gpu, K, True)
     assert torch.equal(i_gpu.cpu().long(), i_from_gpu_logits)
-    _, i_ref = O.route_topk(logits_ref, 8, True)
+    _, i_ref = O.route_topk(logits_ref, K, True)
     diff_rows = (i_gpu.cpu().long() != i_ref).any(dim=1).nonzero().flatten()
     srt = torch.sort(logits_ref, dim=1, descending=True).values
-    gaps = (srt[:, :8] - srt[:, 1:9])          # margins that decide order and membership
+    gaps = (srt[:, :K] - srt[:, 1:K + 1])          # margins that decide order and membership
     for r in diff_rows.tolist():
         assert gaps[r].min().item() < 1e-4, f"row {r} differs without a near-tie"
-    assert len(diff_rows) <= 8
+    print(f"[info] {name}: {len(diff_rows)} of {cfg.tokens} tokens routed differently from the CPU evaluation "
+          f"(all on margins below 1e-4)", flush=True)
+    assert len(diff_rows) <= cfg.tokens // 512
 
 
 def test_sort_expert_order_hint(dev):

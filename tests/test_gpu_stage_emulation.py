@@ -56,8 +56,9 @@ def _rope(x, theta=1e6):
     return torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).to(x.dtype)
 
 
-def _layer_forward(x, p, cfg, hip: bool):
-    """x [B,S,dim] -> [B,S,dim].  hip=True: RMSNorms and the MoE block on the HIP kernels."""
+def _layer_forward(x, p, cfg, hip: bool, top_idx=None):
+    """x [B,S,dim] -> [B,S,dim].  hip=True: RMSNorms and the MoE block on the HIP kernels.  top_idx
+    (oracle side only): route with these expert indices instead of the oracle's own selection."""
     dim, n_heads, n_kv, hd, E, I, K = cfg
     B, S, _ = x.shape
     norm = (lambda t, w: F_.rmsnorm(t, w, 1e-6)) if hip else (lambda t, w: O.rmsnorm(t, w, 1e-6))
@@ -74,7 +75,7 @@ def _layer_forward(x, p, cfg, hip: bool):
         y = F_.moe_block(x2, p["ffn_norm"], p["w_gate"], None, p["w1"], p["w2"], p["w3"], top_k=K, route_norm=True)
     else:
         y, _ = O.moe_block(x2, p["ffn_norm"], p["w_gate"], None, p["w1"], p["w2"], p["w3"], K, True,
-                           compute_dtype=torch.float32)
+                           compute_dtype=torch.float32, top_idx=top_idx)
     return y.reshape(B, S, dim)
 
 
@@ -129,33 +130,58 @@ def test_reduced_stage_against_cpu_oracle(dev):
     layers = [_init_layer(gen, shapes, dtype) for _ in range(2)]
     xs = [torch.randn(B, S, cfg[0], generator=gen).to(dtype) for _ in range(MB)]
 
+    # the device runs first and its routing decisions are recorded, in call order (1F1B on one
+    # rank: microbatch by microbatch, layer 0 then layer 1)
+    from piper_amd import ops
+    chosen = []
+    real_topk = ops.route_topk
+
+    def recording_topk(*a, **kw):
+        scores, idx = real_topk(*a, **kw)
+        chosen.append(idx.cpu())
+        return scores, idx
+
+    store, ex, names = _build(layers, cfg, dev, dtype)
+    ops.route_topk = recording_topk
+    try:
+        out = ex.run(one_f_one_b(MB, [0, 1]), [x.to(dev) for x in xs])
+        torch.cuda.synchronize()
+    finally:
+        ops.route_topk = real_topk
+    assert len(chosen) == 2 * MB
+
+    # The oracle routes every token as the device did.  End to end the bf16 stage feeds its routers
+    # activations that differ from the fp32 oracle's by bf16 rounding (attention, previous layer), so
+    # a few tokens on a near-tie would otherwise choose another expert and move their contribution
+    # between expert gradients, which no tolerance on a gradient can tell from a wrong scale.
     ref = [{k: v.clone().float().requires_grad_(True) for k, v in l.items()} for l in layers]
     ref_losses = []
-    for x in xs:
+    flips = 0
+    for mb, x in enumerate(xs):
         h = x.float()
-        for p in ref:
-            h = _layer_forward(h, p, cfg, False)
+        for li, p in enumerate(ref):
+            idx = chosen[2 * mb + li]
+            with torch.no_grad():      # how many tokens the oracle alone would have routed differently
+                own = _layer_forward(h, p, cfg, False)
+            h_next = _layer_forward(h, p, cfg, False, top_idx=idx)
+            flips += int((own - h_next.detach()).abs().amax(dim=-1).gt(0).sum())
+            h = h_next
         loss = h.sum()
         loss.backward()
         ref_losses.append(loss.detach())
+    print(f"[info] tokens routed differently by the fp32 oracle on its own: {flips} of {2 * MB * B * S}", flush=True)
 
-    store, ex, names = _build(layers, cfg, dev, dtype)
-    out = ex.run(one_f_one_b(MB, [0, 1]), [x.to(dev) for x in xs])
-    torch.cuda.synchronize()
     for got, want in zip(out["losses"], ref_losses):
         assert abs(got.item() - want.item()) <= max(4 * BF16_TOL * abs(want.item()), 2.0)
-    # End to end the bf16 stage feeds its routers activations that differ from the fp32 oracle's by
-    # bf16 rounding (attention, previous layer), so a few near-tie tokens choose another expert and
-    # their contribution moves between expert gradients: the bound on the normalised maximum error
-    # is wide here; the per-kernel 2e-2 parity is tested on identical inputs in the other test files.
+    # two layers deep, gradients accumulated over three microbatches: 4x the single-kernel bound
     for ubid in (0, 1):
         b = store.buckets[ubid]
         for (p, off, n, shape), name in zip(b.param_view_specs, names):
             got = b.flat_grads[off:off + n].view(shape)
-            assert rel_err(got, ref[ubid][name].grad) <= 0.25, (ubid, name)
+            assert rel_err(got, ref[ubid][name].grad) <= 4 * BF16_TOL, (ubid, name)
         gb = store.buckets[f"gate{ubid}"]
         got = gb.flat_grads[: math.prod(shapes["w_gate"])].view(shapes["w_gate"])
-        assert rel_err(got, ref[ubid]["w_gate"].grad) <= 0.3
+        assert rel_err(got, ref[ubid]["w_gate"].grad) <= 4 * BF16_TOL
 
 
 def test_full_size_stage_properties(dev):
