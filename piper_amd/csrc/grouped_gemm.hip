@@ -400,10 +400,10 @@ __host__ __device__ __forceinline__ int padded_start(int start, int e) {
 }
 
 // Division of a non-negative int32 by a divisor fixed per launch without the ~25 instructions of
-// the general integer division: a shift for powers of two, otherwise multiply-high by
-// floor(2^(31+s)/d)+1 and shift by s-1 with s = ceil(log2 d) (exact for 0 <= n < 2^31).
+// the general integer division: multiply-high by 2^(32-s) for d = 2^s, otherwise by
+// floor(2^(31+s)/d)+1 followed by a shift by s-1 with s = ceil(log2 d) (exact for 0 <= n < 2^31).
 struct FastDiv {
-  uint32_t mul;    // 0: divisor is 2^shift
+  uint32_t mul;    // 0: divisor is 1
   int32_t shift;
 };
 inline FastDiv make_fastdiv(int64_t d) {
@@ -411,14 +411,18 @@ inline FastDiv make_fastdiv(int64_t d) {
   if (d <= 1) return f;
   int s = 0;
   while (((int64_t)1 << s) < d) ++s;
-  if (((int64_t)1 << s) == d) { f.shift = s; return f; }
+  if (((int64_t)1 << s) == d) { f.mul = 1u << (32 - s); return f; }   // mulhi by 2^(32-s) is the shift by s
   f.mul = (uint32_t)((((uint64_t)1 << (31 + s)) / (uint64_t)d) + 1u);
   f.shift = s - 1;
   return f;
 }
+// No branch on the divisor's kind (it would sit between the MFMAs of the loops that divide per lane):
+// the product is always formed and a mask picks n itself for a divisor of 1.
 __device__ __forceinline__ int fastdiv(int n, const FastDiv f) {
   const uint32_t u = (uint32_t)n;
-  return (int)((f.mul ? __umulhi(u, f.mul) : u) >> f.shift);
+  const uint32_t q = __umulhi(u, f.mul) >> f.shift;
+  const uint32_t keep = f.mul == 0u ? 0xffffffffu : 0u;
+  return (int)((u & keep) | (q & ~keep));
 }
 
 struct RaggedMParams {
@@ -1333,6 +1337,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
   // division by the map divisor happens per lane as well (a chain of scalar instructions per row
   // -- compare, select, divide, 64-bit multiply -- cost this loop 600 of its 2,400 cycles per k-tile).
   int rows_n[NR];
+  int slot_v[LMN];
   auto fetch_rows = [&](const Unit& t, int kt) {
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
@@ -1367,12 +1372,21 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
       dma16(ok ? src : (const void*)g_zero16, is_kc + piece * 1024);
     } else {
       const int i = piece - LKC;
+      const bool ok = is_real && (is_k0 + mn_krow[i] < ld.rows);
+      const void* src = ld.r_base + (int64_t)fastdiv(slot_v[i], p.map_div) * ldr + mn_cofs[i];
+      dma16(ok ? src : (const void*)g_zero16, is_mn + i * 1024);
+    }
+  };
+  // this lane's row map entries for the slot about to be requested, out of the scalar registers:
+  // done at the top of a k-tile, where the wave waits for its first fragments anyway (scalar loads
+  // and LDS reads share a counter, and a scalar result can only be awaited by draining it)
+  auto take_rows = [&]() {
+#pragma unroll
+    for (int i = 0; i < LMN; ++i) {
       int slot = rows_n[i * MN_RPI];
 #pragma unroll
       for (int r = 1; r < MN_RPI; ++r) slot = mn_rsel == r ? rows_n[i * MN_RPI + r] : slot;
-      const bool ok = is_real && (is_k0 + mn_krow[i] < ld.rows);
-      const void* src = ld.r_base + (int64_t)fastdiv(slot, p.map_div) * ldr + mn_cofs[i];
-      dma16(ok ? src : (const void*)g_zero16, is_mn + i * 1024);
+      slot_v[i] = slot;
     }
   };
   // the first NS-1 k-tiles of unit t into the stages from `first_stage` on
@@ -1382,6 +1396,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
     for (int s = 0; s < NS - 1; ++s) {
       issue_setup(s, first_stage + s >= NS ? first_stage + s - NS : first_stage + s);
       fetch_rows(t, s);
+      take_rows();
 #pragma unroll
       for (int i = 0; i < L; ++i) issue_piece(i);
     }
@@ -1444,13 +1459,14 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
         if (of_next && slot == nkt) ld = load_src(nxt_u);
         const int tgt = cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1;
         issue_setup(of_next ? slot - nkt : slot, tgt);
+        take_rows();
+        // row map entries of the slot after this one: on their way during this tile's MFMAs
+        if (chained && slot + 1 >= nkt) fetch_rows(nxt_u, slot + 1 - nkt);
+        else fetch_rows(cur_u, slot + 1);
         const char* st = smem + cur * STAGE;
         const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
         mma_ktile<BK, TM, TN, A_KC, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN, f0, acc,
                                                      [&](int piece) { issue_piece(piece); });
-        // row map entries of the slot after this one
-        if (chained && slot + 1 >= nkt) fetch_rows(nxt_u, slot + 1 - nkt);
-        else fetch_rows(cur_u, slot + 1);
         cur = cur + 1 == NS ? 0 : cur + 1;
       }
     }
