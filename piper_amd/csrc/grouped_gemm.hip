@@ -11,6 +11,7 @@
 #include <atomic>
 #include <initializer_list>
 #include <mutex>
+#include <type_traits>
 
 namespace {
 
@@ -55,6 +56,25 @@ __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
                :: "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr)
                : "memory");
 }
+// The same load with the address split into a wave-uniform 64-bit base (scalar registers) and a
+// 32-bit byte offset per lane: a k-loop then advances one scalar pointer per operand and k-tile
+// instead of forming a 64-bit address per lane and load.  The LDS destination is lds_base + IMM.
+template <int IMM>
+__device__ __forceinline__ void dma16_s(uint32_t voff, const void* sbase, uint32_t lds_base) {
+  asm volatile("s_add_i32 m0, %0, %3\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(lds_base), "v"(voff), "s"(sbase), "n"(IMM)
+               : "memory", "scc");
+}
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{}) in order
+template <int I0, int N, typename F>
+__device__ __forceinline__ void static_for_impl(F&& f) {
+  if constexpr (I0 < N) {
+    f(std::integral_constant<int, I0>{});
+    static_for_impl<I0 + 1, N>(f);
+  }
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) { static_for_impl<0, N>(f); }
 template <int N>
 __device__ __forceinline__ void wait_dma() {
   asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
@@ -62,6 +82,15 @@ __device__ __forceinline__ void wait_dma() {
 __device__ __forceinline__ void block_barrier() {
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+}
+// A wave-uniform 64-bit value that the compiler could not prove uniform: into scalar registers.
+__device__ __forceinline__ int64_t uniform_i64(int64_t x) {
+  const uint64_t v = (uint64_t)x;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ const char* uniform_ptr(const char* p) {
+  return (const char*)(uintptr_t)uniform_i64((int64_t)(uintptr_t)p);
 }
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
   return (uint32_t)(uintptr_t)(lds_ptr_t)p;
@@ -405,9 +434,10 @@ __host__ __device__ __forceinline__ int padded_start(int start, int e) {
 struct FastDiv {
   uint32_t mul;    // 0: divisor is 1
   int32_t shift;
+  int64_t d;       // the divisor itself (host side checks)
 };
 inline FastDiv make_fastdiv(int64_t d) {
-  FastDiv f = {0u, 0};
+  FastDiv f = {0u, 0, d < 1 ? 1 : d};
   if (d <= 1) return f;
   int s = 0;
   while (((int64_t)1 << s) < d) ++s;
@@ -561,32 +591,27 @@ __device__ __forceinline__ void mma_ktile(const char* At, const char* Bt, const 
   // operands the caller has made visible before this call
   Frags<TM, TN> f[2];
   f[0] = f0;
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    __builtin_amdgcn_sched_barrier(0);
-    const bool last = ks + 1 == KS;
+  // issue_one receives the load's index as a compile-time constant (std::integral_constant)
+  static_for<NM>([&](auto idx_c) {
+    constexpr int idx = decltype(idx_c)::value;
+    constexpr int ks = idx / (TM * TN), m = idx % (TM * TN), i = m / TN, j = m % TN;
+    constexpr bool last = ks + 1 == KS;
+    constexpr int ksn = last ? 0 : ks + 1;
     const char* An = last ? At_next : At;
     const char* Bn = last ? Bt_next : Bt;
-    const int ksn = last ? 0 : ks + 1;
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[ks & 1].b[j], f[ks & 1].a[i], acc[i][j], 0, 0, 0);
-        // the sched barriers pin one fragment read of the next k-step (B first: the next
-        // k-step starts with row 0) and at most one load behind each MFMA
-        __builtin_amdgcn_sched_barrier(0);
-        const int m = i * TN + j;
-        if (m < TN)
-          f[(ks + 1) & 1].b[m] = B_KC ? frag_kc<BK>(Bn, wcol0 + 32 * m, ksn, lane) : frag_mn<BCOLS>(Bn, wcol0 + 32 * m, ksn, lane);
-        else if (m < TN + TM)
-          f[(ks + 1) & 1].a[m - TN] = A_KC ? frag_kc<BK>(An, wrow0 + 32 * (m - TN), ksn, lane)
-                                           : frag_mn<ACOLS>(An, wrow0 + 32 * (m - TN), ksn, lane);
-        const int idx = (ks * TM + i) * TN + j;
-        if (idx % EVERY == EVERY - 1 && idx / EVERY < L) issue_one(idx / EVERY);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-  }
+    if constexpr (m == 0) __builtin_amdgcn_sched_barrier(0);
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[ks & 1].b[j], f[ks & 1].a[i], acc[i][j], 0, 0, 0);
+    // the sched barriers pin one fragment read of the next k-step (B first: the next
+    // k-step starts with row 0) and at most one load behind each MFMA
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (m < TN)
+      f[(ks + 1) & 1].b[m] = B_KC ? frag_kc<BK>(Bn, wcol0 + 32 * m, ksn, lane) : frag_mn<BCOLS>(Bn, wcol0 + 32 * m, ksn, lane);
+    else if constexpr (m < TN + TM)
+      f[(ks + 1) & 1].a[m - TN] = A_KC ? frag_kc<BK>(An, wrow0 + 32 * (m - TN), ksn, lane)
+                                       : frag_mn<ACOLS>(An, wrow0 + 32 * (m - TN), ksn, lane);
+    if constexpr (idx % EVERY == EVERY - 1 && idx / EVERY < L) issue_one(std::integral_constant<int, idx / EVERY>{});
+    __builtin_amdgcn_sched_barrier(0);
+  });
   f0 = f[0];
 }
 
@@ -646,49 +671,55 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   }
   int par = 0;
 
-  // ---- lane constants of the loaders
-  int a_kofs[LA];
+  // ---- lane constants of the loaders: byte offsets of a lane's 16 bytes from a wave-uniform base
+  uint32_t a_kofs[LA];
 #pragma unroll
-  for (int i = 0; i < LA; ++i) { int r; kc_slot<BK>(wave * LA + i, lane, r, a_kofs[i]); }
-  int32_t b_loff[LB];     // element offset inside the expert's weight tile
-  int b_mat[LB];
+  for (int i = 0; i < LA; ++i) { int r, k; kc_slot<BK>(wave * LA + i, lane, r, k); a_kofs[i] = (uint32_t)k * 2u; }
+  // EPI_SWIGLU: the rows of a wave's B pieces are 32 consecutive tile rows, i.e. 32 gate rows
+  // (even waves) or 32 up rows (odd waves): a wave reads one of the two matrices only
+  static_assert(EPI != EPI_SWIGLU || (B_KC && LB * RPI == 32), "a wave's B pieces are one 32-row group");
+  uint32_t voffB[LB];
 #pragma unroll
   for (int i = 0; i < LB; ++i) {
-    b_mat[i] = 0;
     if (B_KC) {
       int r, kofs;
       kc_slot<BK>(wave * LB + i, lane, r, kofs);
       int n = r;
-      if (EPI == EPI_SWIGLU) { b_mat[i] = (r >> 5) & 1; n = (r >> 6) * 32 + (r & 31); }
-      b_loff[i] = (int32_t)(n * p.ldb + kofs);
+      if (EPI == EPI_SWIGLU) n = (r >> 6) * 32 + (r & 31);
+      voffB[i] = (uint32_t)(n * (int)p.ldb + kofs) * 2u;
     } else {
       int krow, cofs;
       mn_slot<BN>(wave * LB + i, lane, krow, cofs);
-      b_loff[i] = (int32_t)(krow * p.ldb + cofs);
+      voffB[i] = (uint32_t)(krow * (int)p.ldb + cofs) * 2u;
     }
   }
   const int kt_per_seg = p.Kseg / BK;
   const int nkt = kt_per_seg * p.nseg;
+  const uint32_t row_bytes = (uint32_t)p.lda * 2u;
+  const uint32_t step_a = BK * 2, step_b = B_KC ? (uint32_t)(BK * 2) : (uint32_t)BK * (uint32_t)p.ldb * 2u;
 
   struct Unit {
     int row0, rows, nt;
     int tcol;            // column of row0 in the transposed outputs
-    int64_t b_base;
-    int64_t a_off[LA];
+    int64_t a_base;      // bytes from the A operand to the unit's first row (0 with a row map)
+    int64_t b_base;      // bytes from the weights to the unit's tile
+    uint32_t voff_a[LA]; // per lane: bytes from a_base to its row and 16-byte chunk
   };
   auto setup = [&](Unit& t, int un) {
     int e, mt, nt;
     locate_unit<BM>(ui, starts, p.E, p.n_tiles, un, e, mt, nt);
     const int s0 = starts[e], s1 = starts[e + 1];
-    t.row0 = s0 + mt * BM;
-    t.rows = min(BM, s1 - t.row0);
-    t.nt = nt;
-    t.tcol = padded_start(s0, e) + mt * BM;
-    t.b_base = (int64_t)e * p.strideB + (B_KC ? (int64_t)nt * BN_OUT * p.ldb : (int64_t)nt * BN);
+    // (all wave-uniform; said again so that the pointers built from them stay in scalar registers)
+    t.row0 = __builtin_amdgcn_readfirstlane(s0 + mt * BM);
+    t.rows = __builtin_amdgcn_readfirstlane(min(BM, s1 - t.row0));
+    t.nt = __builtin_amdgcn_readfirstlane(nt);
+    t.tcol = __builtin_amdgcn_readfirstlane(padded_start(s0, e) + mt * BM);
+    t.b_base = uniform_i64(((int64_t)e * p.strideB + (B_KC ? (int64_t)nt * BN_OUT * p.ldb : (int64_t)nt * BN)) * 2);
+    t.a_base = p.row_map ? (int64_t)0 : uniform_i64((int64_t)t.row0 * p.lda * 2);
 #pragma unroll
     for (int i = 0; i < LA; ++i) {
       const int rbase = (wave * LA + i) * RPI;     // first tile row of this dma16 (wave-uniform)
-      int64_t src;
+      int src;
       if (p.row_map) {
         int sel = 0;
 #pragma unroll
@@ -699,61 +730,87 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
         }
         src = fastdiv(sel, p.map_div);
       } else {
-        src = t.row0 + min(rbase + lane / CPR, t.rows - 1);
+        src = min(rbase + lane / CPR, t.rows - 1);
       }
-      t.a_off[i] = src * p.lda + a_kofs[i];
+      t.voff_a[i] = (uint32_t)src * row_bytes + a_kofs[i];
     }
   };
 
-  // DMA of k-tile `kt` of unit `t` into ring stage `stage`: piece 0..LA-1 = A, LA..L-1 = B
-  int is_k0 = 0, is_seg = 0;
-  uint32_t is_a = 0, is_b = 0;
-  auto issue_setup = [&](int kt, int stage) {
-    is_seg = kt >= kt_per_seg ? 1 : 0;
-    is_k0 = (kt - is_seg * kt_per_seg) * BK;
-    is_a = lds_addr(smem + stage * STAGE) + (wave * LA) * 1024;
-    is_b = lds_addr(smem + stage * STAGE + A_BYTES) + (wave * LB) * 1024;
+  // ---- the loader: requests k-tiles in the order the k-loops consume them, NS-1 tiles ahead.
+  // Its position is two wave-uniform pointers (A rows and weights at the current k) that advance
+  // by a constant per k-tile, plus the lanes' offsets of the unit it is in.  At the end of a unit
+  // it moves on to the next unit if that is known by then (the k-loop then never waits for the
+  // first tiles of a unit); otherwise it stays on a tile of the finished unit (requests that land
+  // in free stages) until the epilogue points it at the next unit.
+  const char* ld_a = nullptr;
+  const char* ld_b = nullptr;
+  int64_t ld_a_base = 0, ld_b_base = 0;
+  uint32_t ld_voff_a[LA];
+  int ld_rem = 0, ld_seg = 0;
+  bool ld_on_next = false, ld_idle = false;
+  auto ld_point = [&](int seg) {
+    ld_a = uniform_ptr(reinterpret_cast<const char*>(seg ? p.A1 : p.A0) + ld_a_base);
+    const bf16_t* B = (EPI == EPI_SWIGLU) ? ((wave & 1) ? p.B1 : p.B0) : (seg ? p.B1 : p.B0);
+    ld_b = uniform_ptr(reinterpret_cast<const char*>(B) + ld_b_base);
+    ld_seg = seg;
+    ld_rem = kt_per_seg;
   };
-  // Every k-tile slot of the loop issues its L loads, so the count of loads in flight does not
-  // depend on where in a unit the loop is: with `real` false (no tile left to fetch) they read a
-  // block of zeros into the stage, which nobody reads before it is filled again.
-  bool is_real = true;
-  auto issue_piece = [&](const Unit& t, int piece) {
-    if (piece < LA) {
-      const bf16_t* A = is_seg ? p.A1 : p.A0;
-      const void* src = A + t.a_off[piece] + is_k0;
-      dma16(is_real ? src : (const void*)g_zero16, is_a + piece * 1024);
-    } else {
-      const int i = piece - LA;
-      const bf16_t* B = (EPI == EPI_SWIGLU) ? (b_mat[i] ? p.B1 : p.B0) : (is_seg ? p.B1 : p.B0);
-      const void* src = B + t.b_base + b_loff[i] + (B_KC ? (int64_t)is_k0 : (int64_t)is_k0 * p.ldb);
-      dma16(is_real ? src : (const void*)g_zero16, is_b + i * 1024);
+  auto ld_take = [&](const Unit& t) {
+    ld_a_base = t.a_base;
+    ld_b_base = t.b_base;
+#pragma unroll
+    for (int i = 0; i < LA; ++i) ld_voff_a[i] = t.voff_a[i];
+    ld_idle = false;
+    ld_point(0);
+  };
+  uint32_t ld_lds_a = 0, ld_lds_b = 0;     // LDS destinations of this wave's pieces in the stage being filled
+  auto ld_target = [&](int stage) {
+    ld_lds_a = lds_addr(smem) + stage * STAGE + wave * (LA * 1024);
+    ld_lds_b = lds_addr(smem) + stage * STAGE + A_BYTES + wave * (LB * 1024);
+  };
+  auto issue_piece = [&](auto piece_c) {
+    constexpr int P = decltype(piece_c)::value;
+    if constexpr (P < LA) dma16_s<P * 1024>(ld_voff_a[P], ld_a, ld_lds_a);
+    else dma16_s<(P - LA) * 1024>(voffB[P - LA], ld_b, ld_lds_b);
+  };
+  Unit cur_u, nxt_u;
+  bool next_known = false;
+  // after the L loads of a k-tile slot
+  auto ld_advance = [&]() {
+    ld_a += step_a;
+    ld_b += step_b;
+    if (--ld_rem == 0) {
+      if (!ld_idle && ld_seg + 1 < p.nseg) {
+        ld_point(ld_seg + 1);
+      } else if (!ld_idle && next_known && !ld_on_next) {
+        ld_on_next = true;
+        ld_take(nxt_u);
+      } else {           // nothing to request: the first tile of the same unit, again and again
+        ld_idle = true;
+        ld_point(0);
+        ld_rem = 1;
+      }
     }
   };
-  auto issue_tile = [&](const Unit& t, int kt, int stage) {
-    issue_setup(kt, stage);
-    is_real = kt < nkt;
-#pragma unroll
-    for (int i = 0; i < L; ++i) issue_piece(t, i);
+  // one k-tile slot outside the MFMA loop
+  auto issue_slot = [&](int stage) {
+    ld_target(stage);
+    static_for<L>([&](auto pc) { issue_piece(pc); });
+    ld_advance();
   };
 
   int st_after = 0;     // stores this wave issued after its latest prefetch
-  Unit cur_u, nxt_u;
   setup(cur_u, unit);
   nxt_u = cur_u;
   int cur = 0;          // ring stage of k-tile 0 of the current unit
+  ld_take(cur_u);
 #pragma unroll
-  for (int s = 0; s < NS - 1; ++s) issue_tile(cur_u, s, s);
+  for (int s = 0; s < NS - 1; ++s) issue_slot(s);
 
-  Unit ld_u = cur_u;    // the unit whose k-tiles are being requested: the current one or, chained, the next
   for (;;) {
     int unit_next = -1;
-    // chained: the k-loop goes on requesting k-tiles past the end of this unit -- the first NS-1
-    // of the next unit -- in the slots where it would otherwise request blocks of zeros.  The next
-    // unit's operands are then in LDS when this unit's epilogue ends, and the epilogue's stores do
-    // not stand between those requests and the first MFMA of the next unit.
-    bool chained = false;
-    ld_u = cur_u;
+    next_known = false;
+    ld_on_next = false;
     const bool wave_has_rows = wm * WTM < cur_u.rows;   // waves whose row slice is empty skip the math
 
     floatx16_t acc[TM][TN];
@@ -764,45 +821,47 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
+    // the unit after this one: one lane works it out from the ticket taken during the previous
+    // unit and leaves it in LDS; everyone reads it behind the barrier below and resolves the
+    // unit's addresses (row map lookups included) before the k-loop, which then holds no
+    // bookkeeping besides the loader's
+    if (tid == 0) lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, ui.total));
     // k-tile 0 has landed once only younger operations are in flight: the younger k-tiles and
     // the stores that the previous epilogue issued after its prefetch
     wait_vm_le((NS - 2) * L + st_after);
     block_barrier();
+    unit_next = __builtin_amdgcn_readfirstlane(sched_box[par ^ 1]);
+    if (unit_next >= 0) setup(nxt_u, unit_next);
+    next_known = unit_next >= 0;
     Frags<TM, TN> f0;     // fragments of the first k-step of the coming k-tile, read one tile ahead
     if (wave_has_rows)
       load_frags<BK, TM, TN, true, B_KC, BM, BN>(f0, smem + cur * STAGE, smem + cur * STAGE + A_BYTES, wm * WTM, wn * WTN, 0, lane);
 
-    for (int kt = 0; kt < nkt; ++kt) {
-      // k-tile kt+1 has to be in LDS before this tile's MFMAs: its first fragments are read
-      // while they run, so that no wave waits for LDS behind the barrier of the next tile
-      // (NS-1+kt tiles have been requested, real or not; all but the NS-3 youngest must be there)
-      if (kt == 0) wait_vm_le((NS - 3) * L + st_after);
-      else wait_dma<(NS - 3) * L>();
-      block_barrier();   // everyone's part of tile kt+1 is in LDS; everyone is done reading tile kt-1
-      if (kt == 0 && tid == 0)         // publish the unit after this one
-        lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, ui.total));
-      if (kt == 1) {                    // the box was written before this k-tile's barrier
-        unit_next = __builtin_amdgcn_readfirstlane(sched_box[par ^ 1]);
-        if (unit_next >= 0) setup(nxt_u, unit_next);
-        chained = unit_next >= 0 && nkt >= NS + 1;
-      }
-      const int slot = kt + NS - 1;                                   // the k-tile slot requested during this tile
-      const bool of_next = chained && slot >= nkt;
-      if (of_next && slot == nkt) ld_u = nxt_u;
-      const int tgt = cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1;   // stage of k-tile kt-1 = kt+NS-1
-      issue_setup(of_next ? slot - nkt : slot, tgt);
-      is_real = of_next || slot < nkt;
+    // k-tile kt+1 has to be in LDS before the MFMAs of k-tile kt: its first fragments are read
+    // while they run, so that no wave waits for LDS behind the barrier of the next tile
+    // (NS-1+kt tiles have been requested; all but the NS-3 youngest must be there)
+    wait_vm_le((NS - 3) * L + st_after);
+    block_barrier();
+    for (int kt = 0;;) {
+      ld_target(cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1);   // the stage of k-tile kt-1 takes k-tile kt+NS-1
       const char* st = smem + cur * STAGE;
       const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
       if (wave_has_rows) {
-        mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN,
-                                                     f0, acc, [&](int piece) { issue_piece(ld_u, piece); });
+        mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN, f0, acc,
+                                                     [&](auto pc) {
+                                                       issue_piece(pc);
+                                                       if constexpr (decltype(pc)::value == L - 1) ld_advance();
+                                                     });
       } else {
-#pragma unroll
-        for (int i = 0; i < L; ++i) issue_piece(ld_u, i);
+        static_for<L>([&](auto pc) { issue_piece(pc); });
+        ld_advance();
       }
       cur = cur + 1 == NS ? 0 : cur + 1;
+      if (++kt == nkt) break;
+      wait_dma<(NS - 3) * L>();
+      block_barrier();   // everyone's part of tile kt+1 is in LDS; everyone is done reading tile kt-1
     }
+    const bool chained = ld_on_next;   // the loader is NS-1 tiles into the next unit already
     block_barrier();   // every wave has finished its fragment reads: the whole ring is free
     const bool has_next = unit_next >= 0;
     // nothing is in flight here, so taking the ticket of the unit after the next one costs
@@ -816,8 +875,10 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
       if (chained) return;
       st_after = 0;
       if (has_next) {
+        ld_on_next = true;
+        ld_take(nxt_u);
 #pragma unroll
-        for (int s = 0; s < NS - 1; ++s) issue_tile(nxt_u, s, cur + s >= NS ? cur + s - NS : cur + s);
+        for (int s = 0; s < NS - 1; ++s) issue_slot(cur + s >= NS ? cur + s - NS : cur + s);
       }
     };
     if (!BWD) prefetch_next();
@@ -1574,7 +1635,11 @@ inline SchedSlot* sched_slot_for_launch() {
 template <int BM, int BN, int BK, int WMW, int WNW, int NS, bool B_KC, int EPI>
 int launch_ragged_m(RaggedMParams p, int64_t A_rows, int kernel_id, hipStream_t s) {
   const int64_t max_units = (pk_ceil_div(A_rows, BM) + p.E) * p.n_tiles;
-  if (max_units > 0x7ffffff0ll || p.ldb * (int64_t)(BN > BK ? BN : BK) > 0x7fffffffll) return PK_ERR_SHAPE;
+  if (max_units > 0x7ffffff0ll || p.ldb * (int64_t)(BN > BK ? BN : BK) * 2 > 0x7fffffffll) return PK_ERR_SHAPE;
+  // a lane addresses its A row by a 32-bit byte offset: from the unit's first row without a row
+  // map, from the operand's first row with one (all the rows that the map can name: under 4 GiB)
+  const int64_t a_span_rows = p.row_map ? pk_ceil_div(A_rows, p.map_div.d) : (int64_t)BM;
+  if (p.lda * 2 > 0x7fffffffll || (a_span_rows + 1) * p.lda * 2 > 0xffffffffll) return PK_ERR_SHAPE;
   if ((int64_t)p.Kseg * p.nseg < 2 * BK) return PK_ERR_SHAPE;   // the k-loop publishes the next unit in its second step
   const int64_t grid = max_units < persistent_grid() ? round_up_xcd(max_units) : persistent_grid();
   p.sched = sched_slot_for_launch();

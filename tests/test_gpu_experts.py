@@ -122,6 +122,52 @@ def test_scaled_backward_matches_combine_bwd_then_dgrad(dev, dtype, counts, H, I
             assert float(dw2[e].abs().max()) == 0.0
 
 
+def _row_tile_boundary_counts(E):
+    """Row counts around the 256-row block tile and the 32 rows that an expert's last row tile can
+    take in on top of it: exact multiples, one above, 31 / 32 / 33 above, short and empty experts."""
+    edge = [256, 257, 287, 288, 289, 255, 1, 0, 544, 545, 320, 33, 32, 31, 512, 513, 543, 800, 300, 270,
+            264, 250, 129, 128, 127, 1056, 1057, 16, 272, 260]
+    counts = [edge[i % len(edge)] for i in range(E)]
+    return counts
+
+
+def test_row_tiles_with_extra_rows_at_block_tile_boundaries(dev):
+    """Forward and input gradient on a launch large enough for the 256-row block tiles (8 waves,
+    whose last row tile per expert takes in up to 32 more rows), with row counts on every side of
+    the tile boundaries, every expert against fp32 matmuls of the same bf16 inputs on the device.
+    The rows past the 256th of an expert's last tile are also compared on their own."""
+    E, H, I = 128, 1024, 512
+    counts = _row_tile_boundary_counts(E)
+    A = sum(counts)
+    print(f"[case] row tile boundaries E={E} A={A} H={H} I={I}", flush=True)
+    g_ = torch.Generator().manual_seed(21)
+    x = torch.randn(A, H, generator=g_).to(torch.bfloat16).to(dev)
+    dy = torch.randn(A, H, generator=g_).to(torch.bfloat16).to(dev)
+    w1 = (torch.randn(E, I, H, generator=g_) * 0.05).to(torch.bfloat16).to(dev)
+    w3 = (torch.randn(E, I, H, generator=g_) * 0.05).to(torch.bfloat16).to(dev)
+    w2 = (torch.randn(E, H, I, generator=g_) * 0.05).to(torch.bfloat16).to(dev)
+    starts = ops.counts_to_starts(torch.tensor(counts, dtype=torch.long, device=dev))
+    y, g, u, h = ops.grouped_swiglu_fwd(x, w1, w2, w3, starts)
+    dx, dg, du = ops.grouped_swiglu_dgrad(dy, w1, w2, w3, g, u, starts)
+    torch.cuda.synchronize()
+    s = 0
+    for e, c in enumerate(counts):
+        if c == 0:
+            continue
+        xe = x[s:s + c].float().requires_grad_(True)
+        ge = xe @ w1[e].float().t()
+        ue = xe @ w3[e].float().t()
+        he = torch.nn.functional.silu(ge) * ue
+        ye = he @ w2[e].float().t()
+        (dxe,) = torch.autograd.grad(ye, xe, dy[s:s + c].float())
+        for name, got, ref in (("g", g, ge), ("u", u, ue), ("h", h, he), ("y", y, ye), ("dx", dx, dxe)):
+            assert rel_err(got[s:s + c], ref) <= BF16_TOL, (name, e, c, rel_err(got[s:s + c], ref))
+            t0 = (c - 1) // 256 * 256      # first row of the expert's last 256-row group
+            if 0 < c - t0 <= 32 and t0 > 0:  # these rows ride along with the tile before them
+                assert rel_err(got[s + t0:s + c], ref[t0:]) <= BF16_TOL, (name, "extra rows", e, c)
+        s += c
+
+
 T_CASES = [
     # ragged around the 8-row padding and the 32-row k-tile, empty experts, one long expert
     ([0, 1, 7, 8, 9, 31, 32, 33, 0, 300, 64, 255], 256, 256),
