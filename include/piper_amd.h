@@ -265,9 +265,13 @@ PK_API int pk_grouped_swiglu_wgrad_scaled(const void* d_out, const void* hs, con
 /* The same pair with one operand of every weight-gradient GEMM K-contiguous (the fused region's
  * path for bf16 with H % 256 == 0 and I % 256 == 0).  pk_grouped_swiglu_dgrad_dh_scaled_t writes
  * d_g, d_u [A,I] as above and, instead of hs, the three transposed copies
- *   d_gT, d_uT, hsT  [I][ldt]  (dtype), element (i, padded_start(e) + r) = row r of expert e,
- *   padded_start(e) = (starts[e] & ~63) + 64*e; the columns from an expert's last row up to the next
- *   multiple of 8 are zero, all other columns between experts are neither written nor read.
+ *   d_gT, d_uT, hsT  [ldt / 32][I][32]  (dtype): the routed rows are laid out along a padded row
+ *   axis of length ldt on which row r of expert e has index padded_start(e) + r,
+ *   padded_start(e) = (starts[e] & ~63) + 64*e; the value of column i at padded index q sits at
+ *   [q / 32][i][q % 32] (for every block of 32 padded rows the I columns, each with its 32 row
+ *   values contiguous: the producer writes and the weight-gradient kernels read whole kilobytes).
+ *   The padded rows from an expert's last row up to the next multiple of 8 are zero, all other
+ *   padded rows between experts are neither written nor read.
  * ldt >= pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype) and a multiple of 64; that query returns
  * 0 when the shape or dtype has no such path (use the entry points above then).
  * pk_grouped_swiglu_wgrad_scaled_t computes the same d_w1, d_w2, d_w3 as

@@ -417,12 +417,14 @@ __device__ __forceinline__ void sched_finish(SchedSlot* slot) {
   }
 }
 
-// Column at which expert e's rows start in a transposed ([width][ldt]) copy of an expert-sorted
-// operand: a multiple of 64 (128 bytes: the 32-row pieces that the producer stores and the 32-deep
-// k-tiles that the consumer loads then never straddle a 64-byte sector; with 16-byte alignment
-// the stores cost the producer 25 % of its time), computed from starts[e] alone.  Expert e owns
-// [padded_start(e), padded_start(e+1)), which holds its rows rounded up to a multiple of 8:
-// round_down64(a + n) + 64 > n.  ldt >= round_up64(A) + 64 * E holds every expert.
+// Transposed copies of an expert-sorted [rows][width] operand, for consumers that want the routed
+// rows contiguous: the rows are placed on a padded row axis on which expert e starts at
+// padded_start(e), a multiple of 64 computed from starts[e] alone, and owns
+// [padded_start(e), padded_start(e+1)), which holds its rows rounded up to a multiple of 8
+// (round_down64(a + n) + 64 > n; an axis of round_up64(A) + 64 * E holds every expert).  The copy
+// is stored in blocks of 32 padded rows, [axis / 32][width][32]: column c at padded row q sits at
+// ((q / 32) * width + c) * 32 + q % 32.  A 32-row chunk of 64 columns that the producer stages is
+// then 4 KB of consecutive memory, and a consumer's 32-deep k-tile of 256 columns 16 KB.
 constexpr int kTransposedAlign = 64;
 __host__ __device__ __forceinline__ int padded_start(int start, int e) {
   return (start & ~(kTransposedAlign - 1)) + kTransposedAlign * e;
@@ -479,9 +481,9 @@ struct RaggedMParams {
   const float* scores;   // SWIGLU_BWD_SCALED: score of sorted row r is scores[row_map[r]]
   float* ds_partial;     // SWIGLU_BWD_SCALED: [ldc / 64][total_rows] partial <unscaled d_h, h>
   int64_t total_rows;
-  // SWIGLU_BWD_SCALED, optional: the three outputs once more, transposed ([ldc][ldt], the routed
-  // rows contiguous) for the weight-gradient kernels that want a K-contiguous operand.  Expert e's
-  // rows start at column padded_start(e); columns up to the next multiple of 8 are zero.
+  // SWIGLU_BWD_SCALED, optional: the three outputs once more, transposed in blocks of 32 padded rows
+  // ([ldt / 32][ldc][32], see padded_start) for the weight-gradient kernels that want a K-contiguous
+  // operand; the padded rows up to the next multiple of 8 after an expert's last row are zero.
   bf16_t* T0;            // d_g^T
   bf16_t* T1;            // d_u^T
   bf16_t* T2;            // (score * h)^T
@@ -503,10 +505,12 @@ struct Stage32 {
   // rows [0, nrows) go to dst[r * ldc + 0..COLS); returns the number of store instructions
   // the wave issued (nrows is wave-uniform).  STREAM: nontemporal stores, for results that neither
   // this nor the next kernels read (weight gradients).
+  // (lane: the caller's lane id; a caller that wants the per-lane addresses formed here, not hoisted
+  // out of its loops into registers that stay live across them, passes a value the compiler cannot
+  // see through)
   template <bool ACC, bool STREAM = false>
-  __device__ static __forceinline__ int flush(const char* buf, bf16_t* dst, int64_t ldc, int nrows) {
+  __device__ static __forceinline__ int flush(const char* buf, bf16_t* dst, int64_t ldc, int nrows, int lane = threadIdx.x & 63) {
     constexpr int RPP = 64 / CH, NP = 32 / RPP;
-    const int lane = threadIdx.x & 63;
     const int lr = lane / CH, lc = lane % CH;
     u32x4_t v[NP];
 #pragma unroll
@@ -533,7 +537,8 @@ struct Stage32 {
     }
     return nrows >= 32 ? NP : nrows <= 0 ? 0 : (nrows + RPP - 1) / RPP;
   }
-  // The staged tile transposed: element (r, c) goes to dstT[c * ldt + r], rows in groups of 8
+  // The staged tile transposed: element (r, c) goes to dstT[c * ldt + r] (ldt = 32 for the blocked
+  // transposed copies), rows in groups of 8
   // (16 bytes per lane): the groups that start below nrows are written, so the caller stages zeros
   // in rows nrows..31 when the columns up to the next multiple of 8 must come out as zeros.  dstT
   // + multiples of ldt must be 16-byte aligned.  The transposing LDS read hands a lane 4
@@ -541,15 +546,15 @@ struct Stage32 {
   // and receives rows 0..3 of column i.  One store instruction covers 16 columns x 32 rows: the
   // four 16-lane groups take the four 8-row groups, so each destination row receives 64
   // contiguous bytes per instruction.  Returns the number of store instructions issued.
-  __device__ static __forceinline__ int flush_t(const char* buf, bf16_t* dstT, int64_t ldt, int nrows) {
-    static_assert(COLS == 64, "four passes of 16 columns");
-    const int lane = threadIdx.x & 63;
+  __device__ static __forceinline__ int flush_t(const char* buf, bf16_t* dstT, int64_t ldt, int nrows, int lane = threadIdx.x & 63) {
+    static_assert(COLS % 16 == 0, "passes of 16 columns");
+    constexpr int NQ = COLS / 16;
     const int i = lane & 15, grp = lane >> 4;
     const int r0 = 8 * grp + (i >> 2), r1 = r0 + 4;
     typedef short shortx8_t __attribute__((ext_vector_type(8)));
-    u32x4_t v[4];
+    u32x4_t v[NQ];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {                    // columns 16q .. 16q+15
+    for (int q = 0; q < NQ; ++q) {                   // columns 16q .. 16q+15
       const int col = 16 * q + 4 * (i & 3);          // first of the 4 columns this lane points at
       const char* p0 = buf + r0 * ROWB + ((((col >> 3) ^ r0) & (CH - 1)) << 4) + (col & 7) * 2;
       const char* p1 = buf + r1 * ROWB + ((((col >> 3) ^ r1) & (CH - 1)) << 4) + (col & 7) * 2;
@@ -559,10 +564,10 @@ struct Stage32 {
     }
     if (8 * grp < nrows) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
+      for (int q = 0; q < NQ; ++q)
         *reinterpret_cast<u32x4_t*>(dstT + (int64_t)(16 * q + i) * ldt + 8 * grp) = v[q];
     }
-    return nrows > 0 ? 4 : 0;
+    return nrows > 0 ? NQ : 0;
   }
 };
 
@@ -636,10 +641,13 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   static_assert(EPI != EPI_SWIGLU_BWD_SCALED || WTN == 64, "one score-gradient partial per 64 columns");
   constexpr bool BWD = EPI == EPI_SWIGLU_BWD || EPI == EPI_SWIGLU_BWD_SCALED;
   constexpr bool SCALED = EPI == EPI_SWIGLU_BWD_SCALED;
+  constexpr bool PP = NW == 8;    // two waves per SIMD: the groups of the ping-pong k-loop
   constexpr int OUT_COLS = (EPI == EPI_SWIGLU) ? WTN / 2 : WTN;   // columns a wave writes per output tensor
   constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;       // output columns per tile
-  using St = Stage32<OUT_COLS>;
   constexpr int RING = NS * STAGE;
+  // the plain epilogue can stage 32 columns at a time where the ring leaves no room for all of them
+  constexpr int SW = (EPI == EPI_PLAIN && RING + NW * 64 * OUT_COLS > 160 * 1024) ? 32 : OUT_COLS;
+  using St = Stage32<SW>;
   static_assert(RING + NW * St::BYTES <= 160 * 1024, "LDS budget");
   __shared__ __attribute__((aligned(1024))) char smem[RING + NW * St::BYTES];
   constexpr int CPR = BK / 8, RPI = 64 / CPR;            // 16-byte chunks per A row, A rows per dma16
@@ -798,14 +806,18 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     static_for<L>([&](auto pc) { issue_piece(pc); });
     ld_advance();
   };
+  // the first k-tiles of the unit the loader points at, into the stages from `first` on
+  auto issue_prologue = [&](int first) {
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s) issue_slot(first + s >= NS ? first + s - NS : first + s);
+  };
 
   int st_after = 0;     // stores this wave issued after its latest prefetch
   setup(cur_u, unit);
   nxt_u = cur_u;
   int cur = 0;          // ring stage of k-tile 0 of the current unit
   ld_take(cur_u);
-#pragma unroll
-  for (int s = 0; s < NS - 1; ++s) issue_slot(s);
+  issue_prologue(0);
 
   for (;;) {
     int unit_next = -1;
@@ -833,36 +845,97 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     unit_next = __builtin_amdgcn_readfirstlane(sched_box[par ^ 1]);
     if (unit_next >= 0) setup(nxt_u, unit_next);
     next_known = unit_next >= 0;
-    Frags<TM, TN> f0;     // fragments of the first k-step of the coming k-tile, read one tile ahead
-    if (wave_has_rows)
-      load_frags<BK, TM, TN, true, B_KC, BM, BN>(f0, smem + cur * STAGE, smem + cur * STAGE + A_BYTES, wm * WTM, wn * WTN, 0, lane);
-
-    // k-tile kt+1 has to be in LDS before the MFMAs of k-tile kt: its first fragments are read
-    // while they run, so that no wave waits for LDS behind the barrier of the next tile
-    // (NS-1+kt tiles have been requested; all but the NS-3 youngest must be there)
-    wait_vm_le((NS - 3) * L + st_after);
-    block_barrier();
-    for (int kt = 0;;) {
-      ld_target(cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1);   // the stage of k-tile kt-1 takes k-tile kt+NS-1
-      const char* st = smem + cur * STAGE;
-      const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
-      if (wave_has_rows) {
-        mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN, f0, acc,
-                                                     [&](auto pc) {
-                                                       issue_piece(pc);
-                                                       if constexpr (decltype(pc)::value == L - 1) ld_advance();
-                                                     });
-      } else {
+    if constexpr (PP) {
+      // Two groups of four waves, one wave of each group on every SIMD, half a k-tile apart: while
+      // one group multiplies a k-tile out of registers (16 MFMAs back to back, nothing else), the
+      // other reads the fragments of its next k-tile from LDS, requests a later k-tile from memory
+      // and does the loader's bookkeeping; a barrier, and they swap.  The matrix pipe of a SIMD
+      // then always has one wave feeding it, and that wave neither waits for LDS nor shares the
+      // instruction issue with its own address arithmetic.
+      //   group 0:  M0 | C0 | M1 | C1 | ...        (M: memory phase, C: compute phase, | barrier)
+      //   group 1:   . | M0 | C0 | M1 | ...
+      // Tile t is read from LDS by group 0 in phase 2t and by group 1 in phase 2t+1; the loads of
+      // tile t+NS-1 go into the stage of tile t-1, which both groups have finished reading when
+      // either of them requests it (a memory phase ends with its LDS reads complete).  A wave's
+      // own loads of tile t+1 have landed when the phase before 2t+2 ends: group 0 waits for them
+      // at the end of C_t, group 1 at the end of M_t.
+      constexpr int KS = BK / 16;
+      Frags<TM, TN> fr[KS];
+      const int grp = wave / (NW / 2);
+      if (grp == 1) block_barrier();
+      for (int kt = 0; kt < nkt; ++kt) {
+        // ---- memory phase
+        ld_target(cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1);   // the stage of k-tile kt-1 takes k-tile kt+NS-1
+        const char* st = smem + cur * STAGE;
+        if (wave_has_rows) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+            load_frags<BK, TM, TN, true, B_KC, BM, BN>(fr[ks], st, st + A_BYTES, wm * WTM, wn * WTN, ks, lane);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         static_for<L>([&](auto pc) { issue_piece(pc); });
         ld_advance();
+        cur = cur + 1 == NS ? 0 : cur + 1;
+        // a wave's own part of tile kt+1 must have landed when the phase before its first read
+        // ends: younger than it are the NS-2 tiles after it and, while tile kt+1 is one of those
+        // requested before the previous epilogue's stores, these stores
+        auto wait_next_tile = [&]() {
+          if (kt <= NS - 3) wait_vm_le((NS - 2) * L + st_after);
+          else wait_dma<(NS - 2) * L>();
+        };
+        if (grp == 1) wait_next_tile();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        block_barrier();
+        // ---- compute phase
+        if (wave_has_rows) {
+          __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+              for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[ks].b[j], fr[ks].a[i], acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_s_setprio(0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (grp == 0) wait_next_tile();
+        block_barrier();
       }
-      cur = cur + 1 == NS ? 0 : cur + 1;
-      if (++kt == nkt) break;
-      wait_dma<(NS - 3) * L>();
-      block_barrier();   // everyone's part of tile kt+1 is in LDS; everyone is done reading tile kt-1
+      if (grp == 0) block_barrier();   // the whole ring is free: every fragment is in registers or used
+    } else {
+      Frags<TM, TN> f0;     // fragments of the first k-step of the coming k-tile, read one tile ahead
+      if (wave_has_rows)
+        load_frags<BK, TM, TN, true, B_KC, BM, BN>(f0, smem + cur * STAGE, smem + cur * STAGE + A_BYTES, wm * WTM, wn * WTN, 0, lane);
+
+      // k-tile kt+1 has to be in LDS before the MFMAs of k-tile kt: its first fragments are read
+      // while they run, so that no wave waits for LDS behind the barrier of the next tile
+      // (NS-1+kt tiles have been requested; all but the NS-3 youngest must be there)
+      wait_vm_le((NS - 3) * L + st_after);
+      block_barrier();
+      for (int kt = 0;;) {
+        ld_target(cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1);   // the stage of k-tile kt-1 takes k-tile kt+NS-1
+        const char* st = smem + cur * STAGE;
+        const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
+        if (wave_has_rows) {
+          mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN, f0, acc,
+                                                       [&](auto pc) {
+                                                         issue_piece(pc);
+                                                         if constexpr (decltype(pc)::value == L - 1) ld_advance();
+                                                       });
+        } else {
+          static_for<L>([&](auto pc) { issue_piece(pc); });
+          ld_advance();
+        }
+        cur = cur + 1 == NS ? 0 : cur + 1;
+        if (++kt == nkt) break;
+        wait_dma<(NS - 3) * L>();
+        block_barrier();   // everyone's part of tile kt+1 is in LDS; everyone is done reading tile kt-1
+      }
+      block_barrier();   // every wave has finished its fragment reads: the whole ring is free
     }
     const bool chained = ld_on_next;   // the loader is NS-1 tiles into the next unit already
-    block_barrier();   // every wave has finished its fragment reads: the whole ring is free
     const bool has_next = unit_next >= 0;
     // nothing is in flight here, so taking the ticket of the unit after the next one costs
     // one round trip on one wave, not a drain of stores
@@ -877,14 +950,15 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
       if (has_next) {
         ld_on_next = true;
         ld_take(nxt_u);
-#pragma unroll
-        for (int s = 0; s < NS - 1; ++s) issue_slot(cur + s >= NS ? cur + s - NS : cur + s);
+        issue_prologue(cur);
       }
     };
     if (!BWD) prefetch_next();
 
     // ---- epilogue, 32 rows of the wave tile at a time through the wave's staging buffer
-    const int lrow = lane & 31, lq = 4 * (lane >> 5);
+    int lane_e = lane;      // opaque: the epilogue's per-lane addresses are formed per unit (see Stage32::flush)
+    asm volatile("" : "+v"(lane_e));
+    const int lrow = lane_e & 31, lq = 4 * (lane_e >> 5);
     const int64_t grow0 = (int64_t)(cur_u.row0 + wm * WTM) * p.ldc;
     const int64_t gcol0 = (int64_t)cur_u.nt * BN_OUT + wn * OUT_COLS;
     // SwiGLU backward: the epilogue reads g and u (and, scaled, the row's combine score through the
@@ -893,7 +967,8 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     // registers allow it).  One vector at a time, as the compiler orders the loop below on its
     // own, costs a wave about 2,000 cycles per vector: a quarter of a 128-row unit's time at 4,096
     // tokens.
-    constexpr int JB = !BWD ? 1 : (TM <= 2 ? TN : 1);     // column tiles per batch
+    constexpr bool LEAN_BWD = BWD && TM > 2;
+    constexpr int JB = !BWD ? 1 : (TM <= 2 || LEAN_BWD ? TN : 1);     // column tiles per batch
     u32x2_t graw[JB][4], uraw[JB][4];
     float sc_chunk[BWD ? TM : 1];
     auto load_gu = [&](int i, int j0) {
@@ -920,6 +995,12 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i) sc_chunk[i] = p.scores[slot[i]];
+        // Every score counts as used here, also those of chunks past the unit's last row, which
+        // nothing reads: a load still pending on some path at the end of the epilogue makes the
+        // compiler wait for ALL vector memory operations where its register is next written, and
+        // that is inside the next unit's k-loop, where such a wait drains the ring of operand loads.
+#pragma unroll
+        for (int i = 0; i < TM; ++i) asm volatile("" :: "v"(sc_chunk[i]));
       } else {
 #pragma unroll
         for (int i = 0; i < TM; ++i) sc_chunk[i] = 1.f;
@@ -956,15 +1037,97 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
         }
       } else if (EPI == EPI_PLAIN) {
         if (crows > 0) {
+          constexpr int JS = SW / 32;      // column tiles staged together
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
+          for (int j0 = 0; j0 < TN; j0 += JS) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-              St::put(sbuf, lrow, 32 * j + 8 * q + lq,
-                      pack4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]));
-          wave_lds_fence();
-          st_after += St::template flush<false>(sbuf, p.O0 + goff, p.ldc, crows);
-          wave_lds_fence();
+            for (int j = j0; j < j0 + JS; ++j)
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                St::put(sbuf, lrow, 32 * (j - j0) + 8 * q + lq,
+                        pack4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]));
+            wave_lds_fence();
+            st_after += St::template flush<false>(sbuf, p.O0 + goff + 32 * j0, p.ldc, crows);
+            wave_lds_fence();
+          }
+        }
+      } else if constexpr (LEAN_BWD) {
+        // EPI_SWIGLU_BWD[_SCALED] with 128 accumulator registers: the packed outputs of 32 columns
+        // at a time, d_g and d_u side by side in the staging buffer, score * h after them
+        using S2 = Stage32<32>;
+        static_assert(2 * S2::BYTES <= St::BYTES, "two 32-column areas in a wave's staging buffer");
+        char* const sb0 = sbuf;
+        char* const sb1 = sbuf + S2::BYTES;
+        float ds = 0.f;
+        if (crows > 0) {
+          const float sc = sc_chunk[i];
+          load_gu(i, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          // the loads must have returned before the next unit's first tiles are requested: a load
+          // behind those requests would wait for all of them
+          const bool transposed = SCALED && p.T0 != nullptr;
+          const bool live = lrow < crows;      // the transposed copies want zeros in the rows past the end
+          const u32x2_t zero2 = {0u, 0u};
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            u32x2_t hsv[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              float dh[4], g[4], u[4], og[4], ou[4], oh[4];
+              unpack4(pack4(sc * acc[i][j][4 * q], sc * acc[i][j][4 * q + 1], sc * acc[i][j][4 * q + 2], sc * acc[i][j][4 * q + 3]), dh);
+              unpack4(graw[j][q], g);
+              unpack4(uraw[j][q], u);
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                const float sg = 1.f / (1.f + __expf(-g[t]));
+                og[t] = dh[t] * u[t] * (sg * (1.f + g[t] * (1.f - sg)));
+                ou[t] = dh[t] * (g[t] * sg);
+                if (SCALED) {
+                  const float hv = (g[t] * sg) * u[t];
+                  ds += acc[i][j][4 * q + t] * hv;
+                  oh[t] = sc * hv;
+                }
+              }
+              const bool dead = transposed && !live;
+              S2::put(sb0, lrow, 8 * q + lq, dead ? zero2 : pack4(og[0], og[1], og[2], og[3]));
+              S2::put(sb1, lrow, 8 * q + lq, dead ? zero2 : pack4(ou[0], ou[1], ou[2], ou[3]));
+              if (SCALED) hsv[q] = dead ? zero2 : pack4(oh[0], oh[1], oh[2], oh[3]);
+            }
+            if (j == TN - 1 && i == TM - 1) {
+              __builtin_amdgcn_sched_barrier(0);
+              prefetch_next();
+            }
+            const int64_t tofs = ((int64_t)((cur_u.tcol + wm * WTM + 32 * i) >> 5) * p.ldc + gcol0 + 32 * j) * 32;
+            wave_lds_fence();
+            st_after += S2::template flush<false>(sb0, p.O0 + goff + 32 * j, p.ldc, crows, lane_e);
+            st_after += S2::template flush<false>(sb1, p.O1 + goff + 32 * j, p.ldc, crows, lane_e);
+            if constexpr (SCALED) {
+              if (transposed) {
+                st_after += S2::flush_t(sb0, p.T0 + tofs, 32, crows, lane_e);
+                st_after += S2::flush_t(sb1, p.T1 + tofs, 32, crows, lane_e);
+              }
+            }
+            wave_lds_fence();
+            if constexpr (SCALED) {
+              if (p.O2 || transposed) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) S2::put(sb0, lrow, 8 * q + lq, hsv[q]);
+                wave_lds_fence();
+                if (p.O2) st_after += S2::template flush<false>(sb0, p.O2 + goff + 32 * j, p.ldc, crows, lane_e);
+                if (transposed) st_after += S2::flush_t(sb0, p.T2 + tofs, 32, crows, lane_e);
+                wave_lds_fence();
+              }
+            }
+          }
+          if (SCALED) {
+            // lanes l and l+32 hold the two column halves of row l % 32
+            ds += __shfl_xor(ds, 32);
+            if (lane_e < 32 && lrow < crows)
+              p.ds_partial[(int64_t)((cur_u.nt * BN + wn * WTN) >> 6) * p.total_rows + cur_u.row0 + wm * WTM + 32 * i + lrow] = ds;
+            st_after += 1;
+          }
+        } else if (i == TM - 1) {
+          prefetch_next();
         }
       } else {   // EPI_SWIGLU_BWD[_SCALED]: acc = d_h; d_g = d_h * u * silu'(g), d_u = d_h * silu(g)
         u32x2_t dg[TN][4], du[TN][4], hs[SCALED ? TN : 1][4];
@@ -1030,8 +1193,9 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
             if (out) st_after += St::template flush<false>(sbuf, out + goff, p.ldc, crows);
             if constexpr (SCALED) {
               if (transposed)
-                st_after += St::flush_t(sbuf, (which == 0 ? p.T0 : which == 1 ? p.T1 : p.T2) + gcol0 * p.ldt + (cur_u.tcol + wm * WTM + 32 * i),
-                                        p.ldt, crows);
+                st_after += St::flush_t(sbuf, (which == 0 ? p.T0 : which == 1 ? p.T1 : p.T2) +
+                                                  ((int64_t)((cur_u.tcol + wm * WTM + 32 * i) >> 5) * p.ldc + gcol0) * 32,
+                                        32, crows);
             }
             wave_lds_fence();
           }
@@ -1263,8 +1427,8 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
 
 // ---- weight gradient with one K-contiguous operand, persistent workgroups.
 // C[e][M,N] (+)= sum over the rows r of expert e of  m-side[r, m] * n-side[r, n], where one side comes
-// from a transposed copy ("T": [width][ldt], the routed rows contiguous, expert e at column
-// padded_start(e), written by the scaled SwiGLU backward) and the other side from rows gathered
+// from a transposed copy ("T": blocks of 32 padded rows, [ldt / 32][width][32], expert e at padded
+// row padded_start(e), written by the scaled SwiGLU backward) and the other side from rows gathered
 // through the row map ("R": x or d_out).  Against wgrad_kernel: the T operand is read with
 // ds_read_b128 instead of the transposing read (the LDS read rate bounds a k-loop whose operands
 // both need it), a workgroup walks units taken from the per-XCD counters, requests the first
@@ -1319,7 +1483,9 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
   const int tiles = (p.M / BM) * n_tiles;
   const int per_expert = tiles * p.nprob;
   const int total = p.E * per_expert;
-  const int64_t ldt = p.ldt, ldr = p.ldr;
+  const int64_t ldr = p.ldr;
+  static_assert(BK == 32, "a k-tile is one 32-row block of the transposed copies");
+  const int64_t t_width = A_KC ? p.M : p.N;     // rows of a block of the transposed copy
 
   // ---- which units this workgroup runs.
   // DYNAMIC: from the per-XCD counters, as in ragged_m_kernel (balances the very uneven experts of
@@ -1357,13 +1523,13 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
   }
 
   // ---- lane constants of the loaders
-  int64_t kc_loff[LKC];   // element offset of this lane's 16 bytes inside a T tile: row * ldt + k
+  int64_t kc_loff[LKC];   // element offset of this lane's 16 bytes inside a T tile: row * 32 + k
   int kc_k[LKC];
 #pragma unroll
   for (int i = 0; i < LKC; ++i) {
     int r;
     kc_slot<BK>(wave * LKC + i, lane, r, kc_k[i]);
-    kc_loff[i] = (int64_t)r * ldt + kc_k[i];
+    kc_loff[i] = (int64_t)r * 32 + kc_k[i];
   }
   int mn_cofs[LMN], mn_krow[LMN];          // column offset and k-row (inside a tile) of this lane's 16 bytes
 #pragma unroll
@@ -1373,7 +1539,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
   struct Unit {
     int e, q, mt, nt;
     int s0, rows, nkt, kcols;    // first sorted row, row count, k-tiles, rows rounded up to 8
-    const bf16_t* t_base;        // T + first tile row * ldt + padded_start(e)
+    const bf16_t* t_base;        // T + the block of padded_start(e), first tile row
     const bf16_t* r_base;        // R + first tile column
   };
   auto setup = [&](Unit& t, int un) {
@@ -1389,7 +1555,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
     t.nkt = (t.rows + BK - 1) / BK;
     t.kcols = (t.rows + 7) & ~7;
     const WgradKcProblem& q = p.prob[t.q];
-    t.t_base = q.T + (int64_t)(A_KC ? t.mt * BM : t.nt * BN) * ldt + padded_start(t.s0, t.e);
+    t.t_base = q.T + ((int64_t)(padded_start(t.s0, t.e) >> 5) * t_width + (A_KC ? t.mt * BM : t.nt * BN)) * 32;
     t.r_base = q.R + (A_KC ? t.nt * BN : t.mt * BM);
   };
   // Flat slots (row map entries) of the R rows of k-tile kt, wave-uniform, fetched with scalar
@@ -1429,7 +1595,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
   auto issue_piece = [&](int piece) {
     if (piece < LKC) {
       const bool ok = is_real && (is_k0 + kc_k[piece] < ld.kcols);
-      const void* src = ld.t_base + kc_loff[piece] + is_k0;
+      const void* src = ld.t_base + kc_loff[piece] + (int64_t)(is_k0 >> 5) * t_width * 32;
       dma16(ok ? src : (const void*)g_zero16, is_kc + piece * 1024);
     } else {
       const int i = piece - LKC;
@@ -1451,7 +1617,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
     }
   };
   // the first NS-1 k-tiles of unit t into the stages from `first_stage` on
-  auto issue_prologue = [&](const Unit& t, int first_stage) {
+  auto issue_prologue = [&](const Unit& t, int first_stage) __attribute__((always_inline)) {
     ld = load_src(t);
 #pragma unroll
     for (int s = 0; s < NS - 1; ++s) {
@@ -1640,7 +1806,7 @@ int launch_ragged_m(RaggedMParams p, int64_t A_rows, int kernel_id, hipStream_t 
   // map, from the operand's first row with one (all the rows that the map can name: under 4 GiB)
   const int64_t a_span_rows = p.row_map ? pk_ceil_div(A_rows, p.map_div.d) : (int64_t)BM;
   if (p.lda * 2 > 0x7fffffffll || (a_span_rows + 1) * p.lda * 2 > 0xffffffffll) return PK_ERR_SHAPE;
-  if ((int64_t)p.Kseg * p.nseg < 2 * BK) return PK_ERR_SHAPE;   // the k-loop publishes the next unit in its second step
+  if ((int64_t)p.Kseg * p.nseg < 2 * BK) return PK_ERR_SHAPE;
   const int64_t grid = max_units < persistent_grid() ? round_up_xcd(max_units) : persistent_grid();
   p.sched = sched_slot_for_launch();
   if (!p.sched) return PK_ERR_UNSUPPORTED;
@@ -1755,6 +1921,13 @@ int simt_ragged_k(const void* A, int64_t lda, const int32_t* a_map, const void* 
 // PK_RM_LOWM_UNITS of the 256-row units, and for the scaled SwiGLU backward.
 #define PK_RM_LOWM 128, 256, 32, 2, 4, 5
 #define PK_RM_LOWM_UNITS 3
+// Experts with fewer than PK_RM_SHORT_ROWS rows on average (the weights then dominate the traffic
+// and are read from HBM by one or two row tiles each): 128 rows, 64-deep k-tiles in a 3-stage ring,
+// so that a weight row contributes 128 contiguous bytes per k-tile.  Measured at 256 rows per
+// expert against the 256x256x32 tiles: gate/up -8 %, down -4 %, d_x -3 %; at 1,024 rows per
+// expert +2 % to +8 %.
+#define PK_RM_SHORT 128, 256, 64, 2, 4, 3
+#define PK_RM_SHORT_ROWS 512
 // Output widths that are a multiple of 128 but not of 256.
 #define PK_RM_ALT 128, 128, 64, 2, 2, 4
 // Weight gradient: 256x256x64 in a 2-stage ring; with fewer than PK_WG_SHORTK_ROWS rows per expert on
@@ -1780,10 +1953,17 @@ int launch_rm(mf::RaggedMParams& p, int64_t A, int64_t N, int kernel_id, hipStre
     // workgroup (then the last round of units runs on a half-empty chip)
     const int64_t big_units = (A / 256 + p.E / 2) * p.n_tiles;
     const bool lowm = big_units < (int64_t)PK_RM_LOWM_UNITS * mf::persistent_grid();
-    // the scaled SwiGLU backward holds three packed outputs per chunk: with 256-row units it does
-    // not fit the register file (measured 2 % slower than 128-row units at 16,384 tokens)
+    // the scaled SwiGLU backward stays on 128-row units: its time goes into the epilogue (loads of g
+    // and u, the arithmetic, six stores per value), which 256-row units do not shorten, and with
+    // 128 accumulator registers that epilogue spills (measured 14 % slower at 16,384 tokens even
+    // with the packed outputs staged 32 columns at a time)
     if (lowm || EPI == mf::EPI_SWIGLU_BWD_SCALED) return mf::launch_ragged_m<PK_RM_LOWM, B_KC, EPI>(p, A, kernel_id, s);
-    if constexpr (EPI != mf::EPI_SWIGLU_BWD_SCALED) return mf::launch_ragged_m<PK_RM_CFG, B_KC, EPI>(p, A, kernel_id, s);
+    if constexpr (EPI != mf::EPI_SWIGLU_BWD_SCALED) {
+      if constexpr (EPI == mf::EPI_SWIGLU || EPI == mf::EPI_PLAIN) {
+        if (A < (int64_t)PK_RM_SHORT_ROWS * p.E) return mf::launch_ragged_m<PK_RM_SHORT, B_KC, EPI>(p, A, kernel_id, s);
+      }
+      return mf::launch_ragged_m<PK_RM_CFG, B_KC, EPI>(p, A, kernel_id, s);
+    }
   }
   const int64_t per_tile_alt = (EPI == mf::EPI_SWIGLU) ? 64 : 128;
   p.n_tiles = (int32_t)(N / per_tile_alt);

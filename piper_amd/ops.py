@@ -286,8 +286,8 @@ def grouped_swiglu_dgrad_dh_scaled(d_out, perm, top_scores, w2, g, u, starts):
 
 
 def transposed_ld(A: int, H: int, I: int, E: int, dtype: torch.dtype) -> int:
-    """Row length of the transposed copies for the K-contiguous weight-gradient kernels, or 0 when
-    the shape / dtype has no such path."""
+    """Padded row count `ldt` of the transposed copies for the K-contiguous weight-gradient kernels
+    (a multiple of 64; a copy is [ldt / 32, I, 32]), or 0 when the shape / dtype has no such path."""
     if dtype not in (torch.float32, torch.bfloat16):
         return 0
     return int(_lib.load().pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype_code(dtype)))
@@ -295,7 +295,9 @@ def transposed_ld(A: int, H: int, I: int, E: int, dtype: torch.dtype) -> int:
 
 def grouped_swiglu_dgrad_dh_scaled_t(d_out, perm, top_scores, w2, g, u, starts):
     """grouped_swiglu_dgrad_dh_scaled with the outputs the weight gradient reads written transposed:
-    returns (d_g, d_u [A,I], d_gT, d_uT, hsT [I, ldt], d_scores [T,K] f32)."""
+    returns (d_g, d_u [A,I], d_gT, d_uT, hsT [ldt/32, I, 32], d_scores [T,K] f32).  A transposed copy
+    holds, for every block of 32 padded rows, the I columns with the block's 32 row values
+    contiguous: element (column i, padded row r) sits at [r // 32, i, r % 32]."""
     require_gpu(d_out)
     E, H, I = w2.shape
     A = perm.numel()
@@ -305,7 +307,7 @@ def grouped_swiglu_dgrad_dh_scaled_t(d_out, perm, top_scores, w2, g, u, starts):
     _check(ldt > 0, "grouped_swiglu_dgrad_dh_scaled_t: shape without a transposed path")
     d_g = torch.empty_like(g)
     d_u = torch.empty_like(u)
-    d_gT, d_uT, hsT = (torch.empty((I, ldt), dtype=g.dtype, device=dev) for _ in range(3))
+    d_gT, d_uT, hsT = (torch.empty((ldt // 32, I, 32), dtype=g.dtype, device=dev) for _ in range(3))
     d_scores = torch.empty((T, K), dtype=torch.float32, device=dev)
     ws_bytes = int(_lib.load().pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes(A, I))
     ws = torch.empty(max(ws_bytes, 4) // 4, dtype=torch.float32, device=dev)
@@ -319,7 +321,7 @@ def grouped_swiglu_wgrad_scaled_t(d_out, hsT, d_gT, d_uT, x, starts, E, *, row_m
                                   d_w1=None, d_w2=None, d_w3=None, accumulate=False, expert_order=None):
     """Weight gradients from the transposed outputs of grouped_swiglu_dgrad_dh_scaled_t."""
     require_gpu(d_out)
-    I, ldt = hsT.shape
+    I, ldt = hsT.shape[1], hsT.shape[0] * 32
     H = d_out.shape[1]
     A = row_map.numel()
     dt, dev = d_out.dtype, d_out.device
