@@ -645,24 +645,34 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   constexpr int OUT_COLS = (EPI == EPI_SWIGLU) ? WTN / 2 : WTN;   // columns a wave writes per output tensor
   constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;       // output columns per tile
   constexpr int RING = NS * STAGE;
-  // the plain epilogue can stage 32 columns at a time where the ring leaves no room for all of them
-  constexpr int SW = (EPI == EPI_PLAIN && RING + NW * 64 * OUT_COLS > 160 * 1024) ? 32 : OUT_COLS;
+  // The epilogue's staging area (32 rows x OUT_COLS per wave).  ALIAS: it is the ring stage that no
+  // k-tile occupies between two units -- NS-1 stages hold the next unit's first k-tiles, the stage
+  // of the last consumed tile is free until the next k-loop requests its tile NS-1, behind two
+  // barriers that every wave reaches after its epilogue -- so the whole LDS can be ring.
+  // Otherwise it lies behind the ring, 32 columns wide for the plain epilogue where the ring
+  // leaves no room for all of them.
+  constexpr bool ALIAS = PP && NW * 64 * OUT_COLS <= STAGE;
+  constexpr int SW = ALIAS ? OUT_COLS : (EPI == EPI_PLAIN && RING + NW * 64 * OUT_COLS > 160 * 1024) ? 32 : OUT_COLS;
   using St = Stage32<SW>;
-  static_assert(RING + NW * St::BYTES <= 160 * 1024, "LDS budget");
-  __shared__ __attribute__((aligned(1024))) char smem[RING + NW * St::BYTES];
+  constexpr int SMEM_BYTES = ALIAS ? RING : RING + NW * St::BYTES;
+  static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
+  __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
   constexpr int CPR = BK / 8, RPI = 64 / CPR;            // 16-byte chunks per A row, A rows per dma16
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WNW, wn = wave % WNW;
-  char* const sbuf = smem + RING + wave * St::BYTES;
+  // staging area while `cur_stage` is the stage of the coming unit's k-tile 0
+  auto staging_area = [&](int cur_stage) -> char* {
+    return ALIAS ? smem + (cur_stage == 0 ? NS - 1 : cur_stage - 1) * STAGE : smem + RING;
+  };
   const const_i32_ptr starts = as_const(p.starts);
   const const_i32_ptr row_map = as_const(p.row_map);
 
   // ---- first unit of this workgroup
   // the next unit, written by one lane, double buffered; it lives in the first bytes of the
   // staging area, which is idle between the first two barriers of a k-loop (nkt >= 2)
-  int* const sched_box = reinterpret_cast<int*>(smem + RING);
+  int* sched_box = reinterpret_cast<int*>(staging_area(0));
   const UnitIndex ui = build_unit_index<BM>(p.starts, p.E, p.n_tiles);
   const int xcd = blockIdx.x % NXCD;
   unsigned grab = 0;                  // lane 0 of wave 0: grab index taken one unit ahead
@@ -837,6 +847,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     // unit and leaves it in LDS; everyone reads it behind the barrier below and resolves the
     // unit's addresses (row map lookups included) before the k-loop, which then holds no
     // bookkeeping besides the loader's
+    sched_box = reinterpret_cast<int*>(staging_area(cur));
     if (tid == 0) lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, ui.total));
     // k-tile 0 has landed once only younger operations are in flight: the younger k-tiles and
     // the stores that the previous epilogue issued after its prefetch
@@ -956,6 +967,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     if (!BWD) prefetch_next();
 
     // ---- epilogue, 32 rows of the wave tile at a time through the wave's staging buffer
+    char* const sbuf = staging_area(cur) + wave * St::BYTES;
     int lane_e = lane;      // opaque: the epilogue's per-lane addresses are formed per unit (see Stage32::flush)
     asm volatile("" : "+v"(lane_e));
     const int lrow = lane_e & 31, lq = 4 * (lane_e >> 5);
@@ -1914,16 +1926,18 @@ int simt_ragged_k(const void* A, int64_t lda, const int32_t* a_map, const void* 
 
 // Tile configurations (BM, BN, BK, waves along M, waves along N, LDS ring stages), chosen by
 // measurement on MI355X with random data and multinomial / Zipf row counts.
-// Ragged-M kernels: 256x256x32 block tiles, 8 waves (128x64 wave tiles), 4-stage 128 KB ring.
+// Ragged-M kernels: 256x256x32 block tiles, 8 waves (128x64 wave tiles), 4-stage 128 KB ring (the
+// epilogue stages its output in the stage that no k-tile occupies between two units).
 #define PK_RM_CFG 256, 256, 32, 2, 4, 4
 #define PK_RM_BN 256
 // Same width with 128 rows and a 5-stage ring: for launches that would give a workgroup fewer than
-// PK_RM_LOWM_UNITS of the 256-row units, and for the scaled SwiGLU backward.
+// PK_RM_LOWM_UNITS of the 256-row units.
 #define PK_RM_LOWM 128, 256, 32, 2, 4, 5
 #define PK_RM_LOWM_UNITS 3
 // Experts with fewer than PK_RM_SHORT_ROWS rows on average (the weights then dominate the traffic
-// and are read from HBM by one or two row tiles each): 128 rows, 64-deep k-tiles in a 3-stage ring,
-// so that a weight row contributes 128 contiguous bytes per k-tile.  Measured at 256 rows per
+// and are read from HBM by one or two row tiles each), and the scaled SwiGLU backward at any size:
+// 128 rows, 64-deep k-tiles in a 3-stage ring, so that a weight row contributes 128 contiguous
+// bytes per k-tile.  Measured at 256 rows per
 // expert against the 256x256x32 tiles: gate/up -8 %, down -4 %, d_x -3 %; at 1,024 rows per
 // expert +2 % to +8 %.
 #define PK_RM_SHORT 128, 256, 64, 2, 4, 3
@@ -1956,8 +1970,10 @@ int launch_rm(mf::RaggedMParams& p, int64_t A, int64_t N, int kernel_id, hipStre
     // the scaled SwiGLU backward stays on 128-row units: its time goes into the epilogue (loads of g
     // and u, the arithmetic, six stores per value), which 256-row units do not shorten, and with
     // 128 accumulator registers that epilogue spills (measured 14 % slower at 16,384 tokens even
-    // with the packed outputs staged 32 columns at a time)
-    if (lowm || EPI == mf::EPI_SWIGLU_BWD_SCALED) return mf::launch_ragged_m<PK_RM_LOWM, B_KC, EPI>(p, A, kernel_id, s);
+    // with the packed outputs staged 32 columns at a time).  64-deep k-tiles in a 3-stage ring
+    // against 32-deep ones in a 5-stage ring: -9 % at 4,096 tokens, -8 % at 16,384.
+    if constexpr (EPI == mf::EPI_SWIGLU_BWD_SCALED) return mf::launch_ragged_m<PK_RM_SHORT, B_KC, EPI>(p, A, kernel_id, s);
+    if (lowm) return mf::launch_ragged_m<PK_RM_LOWM, B_KC, EPI>(p, A, kernel_id, s);
     if constexpr (EPI != mf::EPI_SWIGLU_BWD_SCALED) {
       if constexpr (EPI == mf::EPI_SWIGLU || EPI == mf::EPI_PLAIN) {
         if (A < (int64_t)PK_RM_SHORT_ROWS * p.E) return mf::launch_ragged_m<PK_RM_SHORT, B_KC, EPI>(p, A, kernel_id, s);

@@ -55,6 +55,10 @@ __global__ __launch_bounds__(kRowThreads) void permute_fwd_kernel(
 }
 
 // out[t,:] = sum_k w[t,k] * rows[inv_perm[t*K+k], :] (+ addend[t,:]) (+ residual[t,:]);  w == nullptr -> 1
+// The K rows of a token lie anywhere in the expert-sorted array, so every term is a round trip to
+// memory behind the load of its index.  Indices and weights of up to KB terms are fetched first
+// (wave-uniform addresses), then the KB row loads are issued together and summed in k order (the
+// same sum, term by term, as one load at a time).
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void gather_reduce_kernel(
     const T* __restrict__ rows, const int32_t* __restrict__ inv_perm,
@@ -62,19 +66,32 @@ __global__ __launch_bounds__(kRowThreads) void gather_reduce_kernel(
     T* __restrict__ out, int64_t H, int K) {
   using IO = RowIO<T, VEC>;
   constexpr int N = PkVec16<T>::N;
+  constexpr int KB = 8;
   const int64_t t = blockIdx.x;
   const int64_t nv = H / IO::N;
   for (int64_t v = threadIdx.x; v < nv; v += kRowThreads) {
     float acc[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) acc[i] = 0.f;
-    for (int k = 0; k < K; ++k) {
-      const int64_t p = inv_perm[t * K + k];
-      const float w = weights ? weights[t * K + k] : 1.f;
-      float f[N];
-      IO::load(rows + p * H, v, f);
+    for (int k0 = 0; k0 < K; k0 += KB) {
+      int64_t p[KB];
+      float w[KB];
 #pragma unroll
-      for (int i = 0; i < IO::N; ++i) acc[i] = fmaf(w, f[i], acc[i]);
+      for (int j = 0; j < KB; ++j) {
+        const int k = min(k0 + j, K - 1);       // past the end: the last term again, not added
+        p[j] = inv_perm[t * K + k];
+        w[j] = weights ? weights[t * K + k] : 1.f;
+      }
+      float f[KB][N];
+#pragma unroll
+      for (int j = 0; j < KB; ++j) IO::load(rows + p[j] * H, v, f[j]);
+#pragma unroll
+      for (int j = 0; j < KB; ++j) {
+        if (k0 + j < K) {
+#pragma unroll
+          for (int i = 0; i < IO::N; ++i) acc[i] = fmaf(w[j], f[j][i], acc[i]);
+        }
+      }
     }
     if (addend) {
 #pragma unroll
