@@ -1930,17 +1930,16 @@ int simt_ragged_k(const void* A, int64_t lda, const int32_t* a_map, const void* 
 // epilogue stages its output in the stage that no k-tile occupies between two units).
 #define PK_RM_CFG 256, 256, 32, 2, 4, 4
 #define PK_RM_BN 256
-// Same width with 128 rows and a 5-stage ring: for launches that would give a workgroup fewer than
-// PK_RM_LOWM_UNITS of the 256-row units.
-#define PK_RM_LOWM 128, 256, 32, 2, 4, 5
-#define PK_RM_LOWM_UNITS 3
-// Experts with fewer than PK_RM_SHORT_ROWS rows on average (the weights then dominate the traffic
-// and are read from HBM by one or two row tiles each), and the scaled SwiGLU backward at any size:
-// 128 rows, 64-deep k-tiles in a 3-stage ring, so that a weight row contributes 128 contiguous
-// bytes per k-tile.  Measured at 256 rows per
-// expert against the 256x256x32 tiles: gate/up -8 %, down -4 %, d_x -3 %; at 1,024 rows per
-// expert +2 % to +8 %.
+// Same width with 128 rows, 64-deep k-tiles in a 3-stage ring (a weight row contributes 128
+// contiguous bytes per k-tile).  For launches that would give a workgroup fewer than
+// PK_RM_LOWM_UNITS of the 256-row units (the last round of units would run on a half-empty chip);
+// for experts with fewer than PK_RM_SHORT_ROWS rows on average, where the weights dominate the
+// traffic and are read from HBM by one or two row tiles each (measured at 256 rows per expert
+// against the 256x256x32 tiles: gate/up -8 %, down -4 %, d_x -3 %; at 1,024 rows per expert +2 %
+// to +8 %); and for the scaled SwiGLU backward at any size (against 32-deep k-tiles in a 5-stage
+// ring: -9 % at 4,096 tokens, -8 % at 16,384).
 #define PK_RM_SHORT 128, 256, 64, 2, 4, 3
+#define PK_RM_LOWM_UNITS 3
 #define PK_RM_SHORT_ROWS 512
 // Output widths that are a multiple of 128 but not of 256.
 #define PK_RM_ALT 128, 128, 64, 2, 2, 4
@@ -1970,16 +1969,10 @@ int launch_rm(mf::RaggedMParams& p, int64_t A, int64_t N, int kernel_id, hipStre
     // the scaled SwiGLU backward stays on 128-row units: its time goes into the epilogue (loads of g
     // and u, the arithmetic, six stores per value), which 256-row units do not shorten, and with
     // 128 accumulator registers that epilogue spills (measured 14 % slower at 16,384 tokens even
-    // with the packed outputs staged 32 columns at a time).  64-deep k-tiles in a 3-stage ring
-    // against 32-deep ones in a 5-stage ring: -9 % at 4,096 tokens, -8 % at 16,384.
-    if constexpr (EPI == mf::EPI_SWIGLU_BWD_SCALED) return mf::launch_ragged_m<PK_RM_SHORT, B_KC, EPI>(p, A, kernel_id, s);
-    if (lowm) return mf::launch_ragged_m<PK_RM_LOWM, B_KC, EPI>(p, A, kernel_id, s);
-    if constexpr (EPI != mf::EPI_SWIGLU_BWD_SCALED) {
-      if constexpr (EPI == mf::EPI_SWIGLU || EPI == mf::EPI_PLAIN) {
-        if (A < (int64_t)PK_RM_SHORT_ROWS * p.E) return mf::launch_ragged_m<PK_RM_SHORT, B_KC, EPI>(p, A, kernel_id, s);
-      }
-      return mf::launch_ragged_m<PK_RM_CFG, B_KC, EPI>(p, A, kernel_id, s);
-    }
+    // with the packed outputs staged 32 columns at a time)
+    if (EPI == mf::EPI_SWIGLU_BWD_SCALED || lowm || A < (int64_t)PK_RM_SHORT_ROWS * p.E)
+      return mf::launch_ragged_m<PK_RM_SHORT, B_KC, EPI>(p, A, kernel_id, s);
+    if constexpr (EPI != mf::EPI_SWIGLU_BWD_SCALED) return mf::launch_ragged_m<PK_RM_CFG, B_KC, EPI>(p, A, kernel_id, s);
   }
   const int64_t per_tile_alt = (EPI == mf::EPI_SWIGLU) ? 64 : 128;
   p.n_tiles = (int32_t)(N / per_tile_alt);
