@@ -77,8 +77,13 @@ def kernel_bytes(cfg) -> dict:
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
 # counters read for a plain device copy of known size.  The numbers and the commands that produced
 # them are in the file named here; a kernel without a committed measurement reports null.
-TRAFFIC_SOURCE = "profiles/bench_hbm_traffic.md"
-MEASURED_TRAFFIC_BYTES = {
+TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.md"
+MEASURED_TRAFFIC_BYTES = {      # (read + written) * 1e6, copied from that file
+    "cfg3": {"swiglu_gate_up": (1060 + 151) * 1e6, "swiglu_down": (484 + 134) * 1e6, "swiglu_dgrad_dh": (801 + 259) * 1e6,
+             "swiglu_dgrad_dx": (975 + 134) * 1e6, "swiglu_wgrad_w13": (343 + 806) * 1e6, "swiglu_wgrad_w2": (207 + 403) * 1e6},
+    "cfg4": {"swiglu_gate_up": (2721 + 605) * 1e6, "swiglu_down": (1292 + 537) * 1e6, "swiglu_dgrad_dh": (2199 + 1020) * 1e6,
+             "swiglu_dgrad_dx": (2601 + 537) * 1e6, "swiglu_wgrad_w13": (1614 + 806) * 1e6, "swiglu_wgrad_w2": (942 + 403) * 1e6},
+    "cfg2": {"pack+adamw": (334 + 680 + 2674 + 2378) * 1e6},
 }
 
 

@@ -185,6 +185,9 @@ PK_API int pk_rmsnorm_bwd(const void* d_y, const void* x, int dtype, const void*
  * bf16 runs on MFMA tiles when H % 128 == 0, I % 128 == 0 and every operand is 16-byte aligned,
  * and on a shape-unrestricted FMA kernel (still HIP, same results to rounding) otherwise; f32 runs on a
  * tiled FMA kernel with no shape restriction.
+ * On the MFMA path an operand whose rows are gathered through a row map (x_rows, d_out) is addressed with
+ * 32-bit byte offsets from its first row: the rows that the map can name (ceil(A / row_map_div) of them)
+ * must span less than 4 GiB, otherwise the call returns PK_ERR_SHAPE and launches nothing.
  */
 
 /* Forward.  x_rows[A_x,H]: when row_map is NULL, row p of the A operand is x_rows[p]
