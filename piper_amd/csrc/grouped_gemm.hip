@@ -225,6 +225,9 @@ __device__ __forceinline__ void mma_tile(const char* At, const char* Bt, int wro
   }
 }
 
+// 1 / (1 + e^-x) with the hardware exponential and reciprocal (each within 1 ulp of fp32; the
+// results are rounded to bf16).  A full-precision division costs ten instructions per value.
+__device__ __forceinline__ float sigmoid_fast(float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
 __device__ __forceinline__ u32x2_t pack4(float a, float b, float c, float d) {
   bf16x4_t v;
   v[0] = (bf16_t)a; v[1] = (bf16_t)b; v[2] = (bf16_t)c; v[3] = (bf16_t)d;
@@ -1037,8 +1040,8 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
                   float g[4], u[4];
                   unpack4(gp, g);
                   unpack4(up, u);
-                  v = pack4((g[0] / (1.f + __expf(-g[0]))) * u[0], (g[1] / (1.f + __expf(-g[1]))) * u[1],
-                            (g[2] / (1.f + __expf(-g[2]))) * u[2], (g[3] / (1.f + __expf(-g[3]))) * u[3]);
+                  v = pack4((g[0] * sigmoid_fast(g[0])) * u[0], (g[1] * sigmoid_fast(g[1])) * u[1],
+                            (g[2] * sigmoid_fast(g[2])) * u[2], (g[3] * sigmoid_fast(g[3])) * u[3]);
                 }
                 St::put(sbuf, lrow, 16 * j + 8 * q + lq, v);
               }
@@ -1091,7 +1094,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
               unpack4(uraw[j][q], u);
 #pragma unroll
               for (int t = 0; t < 4; ++t) {
-                const float sg = 1.f / (1.f + __expf(-g[t]));
+                const float sg = sigmoid_fast(g[t]);
                 og[t] = dh[t] * u[t] * (sg * (1.f + g[t] * (1.f - sg)));
                 ou[t] = dh[t] * (g[t] * sg);
                 if (SCALED) {
@@ -1161,7 +1164,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
               unpack4(uraw[j % JB][q], u);
 #pragma unroll
               for (int t = 0; t < 4; ++t) {
-                const float sg = 1.f / (1.f + __expf(-g[t]));
+                const float sg = sigmoid_fast(g[t]);
                 og[t] = dh[t] * u[t] * (sg * (1.f + g[t] * (1.f - sg)));
                 ou[t] = dh[t] * (g[t] * sg);
                 if (SCALED) {
