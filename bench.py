@@ -273,7 +273,7 @@ def region_result(cfg, steps: int, warmup: int) -> dict:
     # the published peaks, moving its algorithmic bytes takes longer than its algorithmic flops
     intensity = flops[dominant] / nbytes[dominant]
     ridge = MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
-    traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name, {}).get(dominant)
+    traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name.split("-")[0], {}).get(dominant)
     if intensity < ridge:
         achieved = nbytes[dominant] / (dom["avg_ms"] * 1e-3) / 1e9
         roof = {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
