@@ -38,6 +38,8 @@ CASES = [
     ([0, 5, 300, 0, 129, 1, 127, 0], 256, 128),
     ([37] * 16, 128, 384),
     ([0, 0, 0, 700], 384, 256),
+    # enough 256-row units per workgroup for the 256x256 tiles, with a reduction of only four k-tiles
+    ([8192, 8192], 128, 1536),
 ]
 
 
@@ -172,6 +174,7 @@ T_CASES = [
     ([0, 1, 7, 8, 9, 31, 32, 33, 0, 300, 64, 255], 256, 256),
     ([700, 0, 0, 2], 512, 256),
     ([256] * 6, 256, 512),
+    ([4096, 3000, 1000, 96], 256, 1536),
 ]
 
 
