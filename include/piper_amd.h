@@ -273,8 +273,9 @@ PK_API int pk_grouped_swiglu_wgrad_scaled(const void* d_out, const void* hs, con
  *   padded_start(e) = (starts[e] & ~63) + 64*e; the value of column i at padded index q sits at
  *   [q / 32][i][q % 32] (for every block of 32 padded rows the I columns, each with its 32 row
  *   values contiguous: the producer writes and the weight-gradient kernels read whole kilobytes).
- *   The padded rows from an expert's last row up to the next multiple of 8 are zero, all other
- *   padded rows between experts are neither written nor read.
+ *   The padded rows from an expert's last row up to the next multiple of 32 (the end of its last
+ *   block) are zero, and pk_grouped_swiglu_wgrad_scaled_t relies on that; all other padded rows
+ *   between experts are neither written nor read.
  * ldt >= pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype) and a multiple of 64; that query returns
  * 0 when the shape or dtype has no such path (use the entry points above then).
  * pk_grouped_swiglu_wgrad_scaled_t computes the same d_w1, d_w2, d_w3 as

@@ -423,8 +423,9 @@ __device__ __forceinline__ void sched_finish(SchedSlot* slot) {
 // Transposed copies of an expert-sorted [rows][width] operand, for consumers that want the routed
 // rows contiguous: the rows are placed on a padded row axis on which expert e starts at
 // padded_start(e), a multiple of 64 computed from starts[e] alone, and owns
-// [padded_start(e), padded_start(e+1)), which holds its rows rounded up to a multiple of 8
-// (round_down64(a + n) + 64 > n; an axis of round_up64(A) + 64 * E holds every expert).  The copy
+// [padded_start(e), padded_start(e+1)), which holds its rows rounded up to a multiple of 32
+// (the range is a multiple of 64 and longer than the row count: round_down64(a + n) + 64 > n; an
+// axis of round_up64(A) + 64 * E holds every expert).  The copy
 // is stored in blocks of 32 padded rows, [axis / 32][width][32]: column c at padded row q sits at
 // ((q / 32) * width + c) * 32 + q % 32.  A 32-row chunk of 64 columns that the producer stages is
 // then 4 KB of consecutive memory, and a consumer's 32-deep k-tile of 256 columns 16 KB.
@@ -486,7 +487,7 @@ struct RaggedMParams {
   int64_t total_rows;
   // SWIGLU_BWD_SCALED, optional: the three outputs once more, transposed in blocks of 32 padded rows
   // ([ldt / 32][ldc][32], see padded_start) for the weight-gradient kernels that want a K-contiguous
-  // operand; the padded rows up to the next multiple of 8 after an expert's last row are zero.
+  // operand; the padded rows up to the next multiple of 32 after an expert's last row are zero.
   bf16_t* T0;            // d_g^T
   bf16_t* T1;            // d_u^T
   bf16_t* T2;            // (score * h)^T
@@ -541,10 +542,9 @@ struct Stage32 {
     return nrows >= 32 ? NP : nrows <= 0 ? 0 : (nrows + RPP - 1) / RPP;
   }
   // The staged tile transposed: element (r, c) goes to dstT[c * ldt + r] (ldt = 32 for the blocked
-  // transposed copies), rows in groups of 8
-  // (16 bytes per lane): the groups that start below nrows are written, so the caller stages zeros
-  // in rows nrows..31 when the columns up to the next multiple of 8 must come out as zeros.  dstT
-  // + multiples of ldt must be 16-byte aligned.  The transposing LDS read hands a lane 4
+  // transposed copies), rows in groups of 8 (16 bytes per lane).  With nrows > 0 all 32 rows are
+  // written: the caller stages zeros in rows nrows..31, and the consumer finds zeros up to the end
+  // of the 32-row block.  dstT + multiples of ldt must be 16-byte aligned.  The transposing LDS read hands a lane 4
   // consecutive rows of one column: within 16 lanes, lane i points at row i/4, columns 4*(i%4)..+3
   // and receives rows 0..3 of column i.  One store instruction covers 16 columns x 32 rows: the
   // four 16-lane groups take the four 8-row groups, so each destination row receives 64
@@ -565,7 +565,7 @@ struct Stage32 {
       const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) shortx4_t*)(p1));
       v[q] = __builtin_bit_cast(u32x4_t, (shortx8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
     }
-    if (8 * grp < nrows) {
+    if (nrows > 0) {
 #pragma unroll
       for (int q = 0; q < NQ; ++q)
         *reinterpret_cast<u32x4_t*>(dstT + (int64_t)(16 * q + i) * ldt + 8 * grp) = v[q];
@@ -1446,10 +1446,9 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kernel(const WgradParams
 // row padded_start(e), written by the scaled SwiGLU backward) and the other side from rows gathered
 // through the row map ("R": x or d_out).  Against wgrad_kernel: the T operand is read with
 // ds_read_b128 instead of the transposing read (the LDS read rate bounds a k-loop whose operands
-// both need it), a workgroup walks units taken from the per-XCD counters, requests the first
-// k-tiles of its next unit before the epilogue of the current one, and its stores do not hold up
-// the next unit's loads.  A_KC: T is the m side (d_w1 = d_g^T x, d_w3 = d_u^T x); otherwise T is the
-// n side (d_w2 = d_out^T (score h)).  The wave grid puts the wider wave-tile side on T.
+// both need it) and the workgroups are persistent.  A_KC: T is the m side (d_w1 = d_g^T x,
+// d_w3 = d_u^T x); otherwise T is the n side (d_w2 = d_out^T (score h)).  The wave grid puts the
+// wider wave-tile side on T.
 struct WgradKcProblem {
   const bf16_t* T;
   const bf16_t* R;
@@ -1469,19 +1468,38 @@ struct WgradKcParams {
   SchedSlot* sched;
 };
 
-template <int BM, int BN, int BK, int WMW, int WNW, int NS, bool A_KC, bool DYNAMIC>
-__global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcParams p) {
+// The kernel: 256x256x32 tiles, 8 waves, 4-stage ring, the ping-pong k-loop of ragged_m_kernel.
+//  * The two waves of a SIMD belong to two groups half a k-tile apart: one reads the fragments of a
+//    whole k-tile from LDS and requests a later k-tile while the other issues its MFMAs back to
+//    back, with the loader's scalar bookkeeping in the issue slots between the first of them.
+//  * The loader's position is scalar: a pointer into the transposed copy that advances by one
+//    32-row block per k-tile (16 KB of consecutive memory per tile, no masking: the producer writes
+//    zeros in an expert's rows up to the end of its last block), the base of the gathered operand,
+//    and an index into the row map; a load is the scalar-base + 32-bit-lane-offset form.  The row
+//    map entries of the slot after the one being requested are fetched with one 16-byte scalar
+//    load per wave and picked up, per lane, one k-tile later.
+//  * Rows of the gathered operand past the expert's end read whatever row the map holds next (a
+//    valid, finite row): they meet the zeros of the transposed copy.
+//  * One lane resolves the unit after the next one -- ticket, expert, row range -- behind its
+//    epilogue's stores and hands it over through LDS at the top of the next unit, so no wave waits
+//    for a chain of scalar loads between two k-loops.
+//  * A workgroup requests the first k-tiles of its next unit before the epilogue of the current one
+//    (or, when the next unit is known in time, as the last requests of the k-loop), and its
+//    stores do not hold up the next unit's loads.
+template <int WMW, int WNW, bool A_KC, bool DYNAMIC>
+__global__ __launch_bounds__(64 * WMW * WNW) void wgrad_pp_kernel(const WgradKcParams p) {
+  constexpr int BM = 256, BN = 256, BK = 32, NS = 4;
   constexpr bool B_KC = !A_KC;
   constexpr int NW = WMW * WNW, NTHREADS = 64 * NW;
+  static_assert(NW == 8, "two groups of four waves");
   constexpr int WTM = BM / WMW, WTN = BN / WNW, TM = WTM / 32, TN = WTN / 32;
   constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE = A_BYTES + B_BYTES;
   constexpr int KC_ROWS = A_KC ? BM : BN, MN_COLS = A_KC ? BN : BM;
   constexpr int KC_OFF = A_KC ? 0 : A_BYTES, MN_OFF = A_KC ? A_BYTES : 0;
   constexpr int LKC = KC_ROWS * BK * 2 / (NTHREADS * 16), LMN = MN_COLS * BK * 2 / (NTHREADS * 16), L = LKC + LMN;
   constexpr int MN_CPR = MN_COLS / 8, MN_RPI = 64 / MN_CPR, NR = LMN * MN_RPI;
-  static_assert(LKC >= 1 && LMN >= 1 && MN_RPI >= 1, "tile too small for the wave grid");
+  static_assert(MN_RPI == 2, "a load of the gathered operand covers two rows, one per half wave");
   static_assert(WTN % 64 == 0, "the epilogue stages 64 columns at a time");
-  static_assert(NS >= 3, "the k-loop reads the next tile's first fragments one tile ahead");
   using St = Stage32<64>;
   constexpr int RING = NS * STAGE;
   static_assert(RING + NW * St::BYTES <= 160 * 1024, "LDS budget");
@@ -1498,170 +1516,206 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
   const int tiles = (p.M / BM) * n_tiles;
   const int per_expert = tiles * p.nprob;
   const int total = p.E * per_expert;
-  const int64_t ldr = p.ldr;
-  static_assert(BK == 32, "a k-tile is one 32-row block of the transposed copies");
-  const int64_t t_width = A_KC ? p.M : p.N;     // rows of a block of the transposed copy
+  const int t_width = A_KC ? p.M : p.N;            // rows of a block of the transposed copy
+  const uint32_t step_kc = (uint32_t)t_width * 64u;  // bytes from one 32-row block to the next
+  const uint32_t ldr_bytes = (uint32_t)p.ldr * 2u;
 
-  // ---- which units this workgroup runs.
-  // DYNAMIC: from the per-XCD counters, as in ragged_m_kernel (balances the very uneven experts of
-  // skewed routing); the next unit is published through LDS, double buffered, in the first bytes
-  // of wave 0's staging buffer (idle while a k-loop runs).
-  // Otherwise statically: round r gives XCD x the units [(r*8 + x) * G8, +G8), one per workgroup
-  // of that XCD (G8 workgroups per XCD), so the workgroups of an XCD work on neighbouring tiles of
-  // the same experts at the same time; the experts come in descending row count (p.order), so the
-  // units of one round cost about the same.  No atomics, no hand-over through LDS: a few per cent
-  // faster when every expert has a few hundred rows.
-  int* const sched_box = reinterpret_cast<int*>(smem + RING);
+  // ---- which units this workgroup runs: from the per-XCD counters (DYNAMIC; balances the very
+  // uneven experts of skewed routing) or statically, round r giving XCD x the units
+  // [(r*8 + x) * G8, +G8), one per workgroup of that XCD, experts in descending row count
+  // (p.order), so the units of a round cost about the same.  Either way lane 0 works out the
+  // description of a unit (UnitDesc) well before the unit starts and hands it over through LDS:
+  // two boxes in the first bytes of wave 0's staging buffer, which is idle between the end of
+  // that wave's epilogue and the end of the next k-loop.
+  struct UnitDesc { int unit, e, q, mt, nt, s0, s1, pad; };
+  UnitDesc* const box = reinterpret_cast<UnitDesc*>(smem + RING);
   const int xcd = blockIdx.x % NXCD, G8 = gridDim.x / NXCD;
   auto unit_at = [&](int r) {
     const int u = (r * NXCD + xcd) * G8 + (int)(blockIdx.x / NXCD);
     return u < total ? u : -1;
   };
+  // lane 0: the unit after the current one (plain scalars: a struct would live in scratch memory)
+  int nx_unit = -1, nx_e = 0, nx_q = 0, nx_mt = 0, nx_nt = 0, nx_s0 = 0, nx_s1 = 0;
+  auto describe = [&](int un) __attribute__((always_inline)) {
+    un = __builtin_amdgcn_readfirstlane(un);     // one lane runs this: scalar arithmetic and scalar loads
+    nx_unit = un;
+    if (un < 0) return;
+    const int rank = un / per_expert;
+    const int rem = un - rank * per_expert;
+    nx_q = rem / tiles;
+    const int tt = rem - nx_q * tiles;
+    nx_mt = tt / n_tiles;
+    nx_nt = tt - nx_mt * n_tiles;
+    nx_e = p.order ? order[rank] : rank;
+    nx_s0 = starts[nx_e];
+    nx_s1 = starts[nx_e + 1];
+  };
+  auto publish = [&](int which) __attribute__((always_inline)) {
+    int* const b = reinterpret_cast<int*>(&box[which]);
+    b[0] = nx_unit; b[1] = nx_e; b[2] = nx_q; b[3] = nx_mt; b[4] = nx_nt; b[5] = nx_s0; b[6] = nx_s1;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  };
   unsigned grab = 0;
   int par = 0, round = 0;
-  int unit;
-  if constexpr (DYNAMIC) {
-    if (tid == 0) {
-      const int first = sched_resolve(p.sched, xcd, sched_grab(p.sched, xcd), total);
-      sched_box[0] = first;
-      if (first >= 0) grab = sched_grab(p.sched, xcd);
+  if (tid == 0) {
+    int first, second = -1;
+    if constexpr (DYNAMIC) {
+      first = sched_resolve(p.sched, xcd, sched_grab(p.sched, xcd), total);
+      if (first >= 0) second = sched_resolve(p.sched, xcd, sched_grab(p.sched, xcd), total);
+      if (second >= 0) grab = sched_grab(p.sched, xcd);
+    } else {
+      first = unit_at(0);
+      if (first >= 0) second = unit_at(1);
     }
-    __syncthreads();
-    unit = __builtin_amdgcn_readfirstlane(sched_box[0]);
-    if (unit < 0) {
-      if (tid == 0) sched_finish(p.sched);
-      return;
-    }
-  } else {
-    unit = unit_at(0);
-    if (unit < 0) return;
+    describe(first);
+    publish(0);
+    describe(second);
   }
-
-  // ---- lane constants of the loaders
-  int64_t kc_loff[LKC];   // element offset of this lane's 16 bytes inside a T tile: row * 32 + k
-  int kc_k[LKC];
-#pragma unroll
-  for (int i = 0; i < LKC; ++i) {
-    int r;
-    kc_slot<BK>(wave * LKC + i, lane, r, kc_k[i]);
-    kc_loff[i] = (int64_t)r * 32 + kc_k[i];
-  }
-  int mn_cofs[LMN], mn_krow[LMN];          // column offset and k-row (inside a tile) of this lane's 16 bytes
-#pragma unroll
-  for (int i = 0; i < LMN; ++i) mn_slot<MN_COLS>(wave * LMN + i, lane, mn_krow[i], mn_cofs[i]);
-  const int mn_rsel = lane / MN_CPR;       // which of the MN_RPI rows of a load this lane fetches
+  __syncthreads();
 
   struct Unit {
     int e, q, mt, nt;
-    int s0, rows, nkt, kcols;    // first sorted row, row count, k-tiles, rows rounded up to 8
-    const bf16_t* t_base;        // T + the block of padded_start(e), first tile row
-    const bf16_t* r_base;        // R + first tile column
+    int s0, rows, nkt;
+    const char* t_ptr;   // the transposed copy at the expert's first block, first tile row
+    const char* r_ptr;   // the gathered operand at the tile's first column
   };
-  auto setup = [&](Unit& t, int un) {
-    const int rank = un / per_expert;
-    const int rem = un - rank * per_expert;
-    t.q = rem / tiles;
-    const int tt = rem - t.q * tiles;
-    t.mt = tt / n_tiles;
-    t.nt = tt - t.mt * n_tiles;
-    t.e = p.order ? order[rank] : rank;
-    t.s0 = starts[t.e];
-    t.rows = starts[t.e + 1] - t.s0;
+  auto take_box = [&](Unit& t, int which) -> int {
+    const int* const b = reinterpret_cast<const int*>(&box[which]);
+    const int un = __builtin_amdgcn_readfirstlane(b[0]);
+    if (un < 0) return un;
+    t.e = __builtin_amdgcn_readfirstlane(b[1]);
+    t.q = __builtin_amdgcn_readfirstlane(b[2]);
+    t.mt = __builtin_amdgcn_readfirstlane(b[3]);
+    t.nt = __builtin_amdgcn_readfirstlane(b[4]);
+    t.s0 = __builtin_amdgcn_readfirstlane(b[5]);
+    t.rows = __builtin_amdgcn_readfirstlane(b[6]) - t.s0;
     t.nkt = (t.rows + BK - 1) / BK;
-    t.kcols = (t.rows + 7) & ~7;
     const WgradKcProblem& q = p.prob[t.q];
-    t.t_base = q.T + ((int64_t)(padded_start(t.s0, t.e) >> 5) * t_width + (A_KC ? t.mt * BM : t.nt * BN)) * 32;
-    t.r_base = q.R + (A_KC ? t.nt * BN : t.mt * BM);
+    t.t_ptr = uniform_ptr(reinterpret_cast<const char*>(
+        q.T + ((int64_t)(padded_start(t.s0, t.e) >> 5) * t_width + (A_KC ? t.mt * BM : t.nt * BN)) * 32));
+    t.r_ptr = uniform_ptr(reinterpret_cast<const char*>(q.R + (A_KC ? t.nt * BN : t.mt * BM)));
+    return un;
   };
-  // Flat slots (row map entries) of the R rows of k-tile kt, wave-uniform, fetched with scalar
-  // loads one tile before they are needed.  No branch and no arithmetic here: rows past the
-  // expert's end read a clamped index and are masked per lane when the load is issued, and the
-  // division by the map divisor happens per lane as well (a chain of scalar instructions per row
-  // -- compare, select, divide, 64-bit multiply -- cost this loop 600 of its 2,400 cycles per k-tile).
-  int rows_n[NR];
-  int slot_v[LMN];
-  auto fetch_rows = [&](const Unit& t, int kt) {
+  Unit cur_u, nxt_u;
+  if (take_box(cur_u, 0) < 0) {
+    if constexpr (DYNAMIC) {
+      if (tid == 0) sched_finish(p.sched);
+    }
+    return;
+  }
+  nxt_u = cur_u;
+
+  // ---- lane constants of the loaders: byte offsets of a lane's 16 bytes
+  uint32_t voff_kc[LKC];      // inside a 32-row block of the transposed copy: (row * 32 + k) * 2
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
-      // load i / MN_RPI of this wave, row i % MN_RPI of the load
-      const int k = kt * BK + (wave * LMN + i / MN_RPI) * MN_RPI + i % MN_RPI;
-      rows_n[i] = row_map[min(t.s0 + k, p.total_rows - 1)];
+  for (int i = 0; i < LKC; ++i) {
+    int r, k;
+    kc_slot<BK>(wave * LKC + i, lane, r, k);
+    voff_kc[i] = (uint32_t)(r * 32 + k) * 2u;
+  }
+  uint32_t mn_cofs[LMN];      // inside a gathered row
+#pragma unroll
+  for (int i = 0; i < LMN; ++i) {
+    int krow, cofs;
+    mn_slot<MN_COLS>(wave * LMN + i, lane, krow, cofs);
+    mn_cofs[i] = (uint32_t)cofs * 2u;
+  }
+  const bool upper = lane >= 32;     // the second of the two rows of a gathered load
+
+  // ---- the loader: requests k-tiles in the order the k-loops consume them, NS-1 tiles ahead, and
+  // moves on to the next unit at the end of one if that unit is known by then; otherwise it
+  // stays on the first tile of the unit it is in (requests that land in stages nobody reads)
+  // until the epilogue points it at the next unit.  rows_n holds the row map entries of the slot
+  // the loader points at.
+  const char* ld_kc = nullptr;
+  const char* ld_kc0 = nullptr;
+  const char* ld_r = nullptr;
+  int ld_map = 0, ld_map0 = 0, ld_rem = 0;
+  bool ld_on_next = false, ld_idle = false, next_known = false;
+  int rows_n[NR];
+  static_assert(NR == 4, "a wave's rows of a k-tile are one 16-byte scalar load");
+  typedef int i32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+  auto fetch_rows = [&]() {
+    const int idx = ld_map + wave * NR;
+    if (idx + NR <= p.total_rows) {
+      const i32x4_a4 v = *reinterpret_cast<const __attribute__((address_space(4))) i32x4_a4*>(row_map + idx);
+      rows_n[0] = v[0]; rows_n[1] = v[1]; rows_n[2] = v[2]; rows_n[3] = v[3];
+    } else {      // the last entries of the row map
+#pragma unroll
+      for (int i = 0; i < NR; ++i) rows_n[i] = row_map[min(idx + i, p.total_rows - 1)];
     }
   };
-  // The unit whose tiles are being requested (the current one, or, towards the end of a k-loop,
-  // the next one), reduced to what the loader needs.
-  struct LoadSrc {
-    int rows, nkt, kcols;
-    const bf16_t* t_base;
-    const bf16_t* r_base;
+  auto ld_enter = [&](const Unit& t) {
+    ld_kc0 = t.t_ptr;
+    ld_map0 = t.s0;
+    ld_r = t.r_ptr;
+    ld_kc = ld_kc0;
+    ld_map = ld_map0;
+    ld_rem = t.nkt;
+    ld_idle = false;
+    if (ld_rem == 0) { ld_idle = true; ld_rem = 1; }    // an expert without rows: nothing to request
   };
-  auto load_src = [](const Unit& t) { return LoadSrc{t.rows, t.nkt, t.kcols, t.t_base, t.r_base}; };
-  LoadSrc ld;
-  uint32_t is_kc = 0, is_mn = 0;
-  int is_k0 = 0;
-  bool is_real = true;
-  auto issue_setup = [&](int kt, int stage) {
-    is_k0 = kt * BK;
-    is_real = kt < ld.nkt;
-    is_kc = lds_addr(smem + stage * STAGE + KC_OFF) + (wave * LKC) * 1024;
-    is_mn = lds_addr(smem + stage * STAGE + MN_OFF) + (wave * LMN) * 1024;
-  };
-  // Every k-tile slot issues its L loads; what lies past the expert's rows reads a block of zeros.
-  auto issue_piece = [&](int piece) {
-    if (piece < LKC) {
-      const bool ok = is_real && (is_k0 + kc_k[piece] < ld.kcols);
-      const void* src = ld.t_base + kc_loff[piece] + (int64_t)(is_k0 >> 5) * t_width * 32;
-      dma16(ok ? src : (const void*)g_zero16, is_kc + piece * 1024);
-    } else {
-      const int i = piece - LKC;
-      const bool ok = is_real && (is_k0 + mn_krow[i] < ld.rows);
-      const void* src = ld.r_base + (int64_t)fastdiv(slot_v[i], p.map_div) * ldr + mn_cofs[i];
-      dma16(ok ? src : (const void*)g_zero16, is_mn + i * 1024);
+  auto ld_advance = [&]() {
+    ld_kc += step_kc;
+    ld_map += BK;
+    if (--ld_rem == 0) {
+      if (!ld_idle && next_known && !ld_on_next) {
+        ld_on_next = true;
+        ld_enter(nxt_u);
+      } else {
+        ld_idle = true;
+        ld_kc = ld_kc0;
+        ld_map = ld_map0;
+        ld_rem = 1;
+      }
     }
   };
-  // this lane's row map entries for the slot about to be requested, out of the scalar registers:
-  // done at the top of a k-tile, where the wave waits for its first fragments anyway (scalar loads
-  // and LDS reads share a counter, and a scalar result can only be awaited by draining it)
-  auto take_rows = [&]() {
+  uint32_t lds_kc = 0, lds_mn = 0;
+  auto ld_target = [&](int stage) {
+    lds_kc = lds_addr(smem) + stage * STAGE + KC_OFF + wave * (LKC * 1024);
+    lds_mn = lds_addr(smem) + stage * STAGE + MN_OFF + wave * (LMN * 1024);
+  };
+  // One slot is requested in two steps.  slot_issue: the lane offsets of the gathered rows come out
+  // of rows_n and the L loads go out to the stage that ld_target named (`between` runs before the
+  // loads: the k-loop reads its fragments there).  slot_advance: the loader moves on and asks for
+  // the next slot's row map entries -- scalar work that the k-loop does between its MFMAs.
+  auto slot_issue = [&](auto&& between) __attribute__((always_inline)) {
+    uint32_t voff_mn[LMN];
 #pragma unroll
     for (int i = 0; i < LMN; ++i) {
-      int slot = rows_n[i * MN_RPI];
-#pragma unroll
-      for (int r = 1; r < MN_RPI; ++r) slot = mn_rsel == r ? rows_n[i * MN_RPI + r] : slot;
-      slot_v[i] = slot;
+      const int slot = upper ? rows_n[i * MN_RPI + 1] : rows_n[i * MN_RPI];
+      voff_mn[i] = (uint32_t)fastdiv(slot, p.map_div) * ldr_bytes + mn_cofs[i];
     }
+    between();
+    static_for<L>([&](auto pc) {
+      constexpr int P = decltype(pc)::value;
+      if constexpr (P < LKC) dma16_s<P * 1024>(voff_kc[P], ld_kc, lds_kc);
+      else dma16_s<(P - LKC) * 1024>(voff_mn[P - LKC], ld_r, lds_mn);
+    });
   };
-  // the first NS-1 k-tiles of unit t into the stages from `first_stage` on
-  auto issue_prologue = [&](const Unit& t, int first_stage) __attribute__((always_inline)) {
-    ld = load_src(t);
+  auto slot_advance = [&]() __attribute__((always_inline)) {
+    ld_advance();
+    fetch_rows();
+  };
+  auto issue_prologue = [&](int first) __attribute__((always_inline)) {
 #pragma unroll
     for (int s = 0; s < NS - 1; ++s) {
-      issue_setup(s, first_stage + s >= NS ? first_stage + s - NS : first_stage + s);
-      fetch_rows(t, s);
-      take_rows();
-#pragma unroll
-      for (int i = 0; i < L; ++i) issue_piece(i);
+      ld_target(first + s >= NS ? first + s - NS : first + s);
+      slot_issue([] {});
+      slot_advance();
     }
   };
 
-  int st_after = 0;     // stores this wave issued after the latest k-tile request
-  Unit cur_u, nxt_u;
-  setup(cur_u, unit);
-  nxt_u = cur_u;
+  int st_after = 0;     // stores this wave issued after its latest prefetch
   int cur = 0;          // ring stage of k-tile 0 of the current unit
-  issue_prologue(cur_u, 0);
+  ld_enter(cur_u);
+  fetch_rows();
+  issue_prologue(0);
 
   for (;;) {
-    int unit_next = -1;
-    bool resolved = false;
-    // chained: the k-loop goes on requesting tiles past the end of this unit -- the first NS-1 of
-    // the next unit -- where it would otherwise request blocks of zeros, so the next unit's
-    // operands are in LDS when this unit's epilogue ends and the stores of the epilogue do not
-    // stand between the requests and the first MFMA.  Needs the next unit to be known NS tiles
-    // before the end (its row map entries are fetched one tile ahead of the request).
-    bool chained = false;
+    next_known = false;
+    ld_on_next = false;
     const int nkt = cur_u.nkt;
-    ld = load_src(cur_u);
     floatx16_t acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -1670,74 +1724,101 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    if (nkt > 0) {
-      wait_vm_le((NS - 2) * L + st_after);     // k-tile 0 has landed: only younger operations are in flight
-      block_barrier();
-      Frags<TM, TN> f0;
-      load_frags<BK, TM, TN, A_KC, B_KC, BM, BN>(f0, smem + cur * STAGE, smem + cur * STAGE + A_BYTES, wm * WTM, wn * WTN, 0, lane);
-      fetch_rows(cur_u, NS - 1);
+    if (tid == 0) publish(par ^ 1);
+    // k-tile 0 has landed once only younger operations are in flight: the younger k-tiles and
+    // the stores that the previous epilogue issued after its prefetch
+    wait_vm_le((NS - 2) * L + st_after);
+    block_barrier();
+    const int unit_next = take_box(nxt_u, par ^ 1);
+    next_known = unit_next >= 0;
+    {
+      // group 0:  M0 | C0 | M1 | C1 | ...        (M: memory phase, C: compute phase, | barrier)
+      // group 1:   . | M0 | C0 | M1 | ...
+      // Tile t is read from LDS by group 0 in phase 2t and by group 1 in phase 2t+1; the loads of
+      // tile t+NS-1 go into the stage of tile t-1, which both groups have finished reading when
+      // either of them requests it (a memory phase ends with its LDS reads complete).  A wave's
+      // own loads of tile t+1 have landed when the phase before 2t+2 ends: group 0 waits for them
+      // at the end of C_t, group 1 at the end of M_t.
+      constexpr int KS = BK / 16;
+      Frags<TM, TN> fr[KS];
+      const int grp = wave / (NW / 2);
+      if (grp == 1) block_barrier();
+      ld_target(cur == 0 ? NS - 1 : cur - 1);     // the stage of k-tile kt-1 takes k-tile kt+NS-1
       for (int kt = 0; kt < nkt; ++kt) {
-        if (kt == 0) wait_vm_le((NS - 3) * L + st_after);
-        else wait_dma<(NS - 3) * L>();
-        block_barrier();   // tile kt+1 is in LDS for everyone; everyone is done reading tile kt-1
-        if constexpr (DYNAMIC) {
-          if (kt == 0 && tid == 0) lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, total));
-          if (kt == 1) {
-            unit_next = __builtin_amdgcn_readfirstlane(sched_box[par ^ 1]);
-            if (unit_next >= 0) setup(nxt_u, unit_next);
-            resolved = true;
-            chained = unit_next >= 0 && nkt >= NS + 1;
-          }
-        } else {
-          if (kt == 0) {     // the scalar loads of the next unit's description run under this tile's MFMAs
-            unit_next = unit_at(round + 1);
-            if (unit_next >= 0) setup(nxt_u, unit_next);
-            resolved = true;
-            chained = unit_next >= 0 && nkt >= NS + 1;
-          }
-        }
-        const int slot = kt + NS - 1;                  // the k-tile slot requested during this tile
-        const bool of_next = chained && slot >= nkt;
-        if (of_next && slot == nkt) ld = load_src(nxt_u);
-        const int tgt = cur + NS - 1 >= NS ? cur - 1 : cur + NS - 1;
-        issue_setup(of_next ? slot - nkt : slot, tgt);
-        take_rows();
-        // row map entries of the slot after this one: on their way during this tile's MFMAs
-        if (chained && slot + 1 >= nkt) fetch_rows(nxt_u, slot + 1 - nkt);
-        else fetch_rows(cur_u, slot + 1);
+        // ---- memory phase
         const char* st = smem + cur * STAGE;
-        const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
-        mma_ktile<BK, TM, TN, A_KC, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN, f0, acc,
-                                                     [&](int piece) { issue_piece(piece); });
+        slot_issue([&] {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+            load_frags<BK, TM, TN, A_KC, B_KC, BM, BN>(fr[ks], st, st + A_BYTES, wm * WTM, wn * WTN, ks, lane);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        const int filled = cur;     // free once both groups have read it: the next slot's target
         cur = cur + 1 == NS ? 0 : cur + 1;
-      }
-    }
-    block_barrier();   // every wave has finished its fragment reads: the whole ring is free
-    if constexpr (DYNAMIC) {
-      if (!resolved) {   // fewer than two k-tiles: the next unit is settled here instead of in the k-loop
-        if (nkt == 0) {
-          if (tid == 0) lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, total));
-          block_barrier();
+        auto wait_next_tile = [&]() {
+          if (kt <= NS - 3) wait_vm_le((NS - 2) * L + st_after);
+          else wait_dma<(NS - 2) * L>();
+        };
+        if (grp == 1) wait_next_tile();
+        // every fragment counts as used here: the compiler then waits for the LDS reads in this
+        // phase, not in front of the MFMAs, where a wait would also cover the scalar loads that
+        // the bookkeeping between the MFMAs has just issued (LDS and scalar loads share a counter)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i) asm volatile("" :: "v"(fr[ks].a[i]));
+#pragma unroll
+          for (int j = 0; j < TN; ++j) asm volatile("" :: "v"(fr[ks].b[j]));
         }
-        unit_next = __builtin_amdgcn_readfirstlane(sched_box[par ^ 1]);
-        if (unit_next >= 0) setup(nxt_u, unit_next);
-        block_barrier();   // the box lies in wave 0's staging buffer, which the epilogue is about to use
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        block_barrier();
+        // ---- compute phase: the MFMAs back to back, the loader's scalar bookkeeping for the next
+        // slot in the issue slots between the first of them
+        __builtin_amdgcn_s_setprio(1);
+        static_for<KS * TM * TN>([&](auto idx_c) {
+          constexpr int idx = decltype(idx_c)::value;
+          constexpr int ks = idx / (TM * TN), i = (idx % (TM * TN)) / TN, j = idx % TN;
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[ks].b[j], fr[ks].a[i], acc[i][j], 0, 0, 0);
+          if constexpr (idx == 0) {
+            __builtin_amdgcn_sched_barrier(0);
+            slot_advance();
+            ld_target(filled);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        });
+        __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (grp == 0) wait_next_tile();
+        block_barrier();
       }
-    } else {
-      if (!resolved) {   // an expert without rows has no k-loop
-        unit_next = unit_at(round + 1);
-        if (unit_next >= 0) setup(nxt_u, unit_next);
-      }
+      if (grp == 0) block_barrier();   // the whole ring is free: every fragment is in registers or used
     }
+    const bool chained = ld_on_next;   // the loader is NS-1 tiles into the next unit already
     const bool has_next = unit_next >= 0;
-    if constexpr (DYNAMIC) {
-      if (has_next && tid == 0) grab = sched_grab(p.sched, xcd);
+    // lane 0: the unit after the next one.  Its expert and row range are scalar loads that return
+    // while this lane's wave stores its tile; they are handed over at the top of the next unit.
+    if (has_next && tid == 0) {
+      int un2;
+      if constexpr (DYNAMIC) {
+        un2 = sched_resolve(p.sched, xcd, grab, total);
+        if (un2 >= 0) grab = sched_grab(p.sched, xcd);
+      } else {
+        un2 = unit_at(round + 2);
+      }
+      describe(un2);
     }
 
-    // the next unit's first tiles, unless the k-loop has requested them already
+    // the next unit's first k-tiles, unless the k-loop has requested them already (then every
+    // store of this epilogue is younger than they are)
     auto prefetch_next = [&]() {
       st_after = 0;
-      if (has_next && !chained) issue_prologue(nxt_u, cur);
+      if (has_next && !chained) {
+        ld_on_next = true;
+        ld_enter(nxt_u);
+        fetch_rows();
+        issue_prologue(cur);
+      }
     };
     // an accumulating epilogue reads the old gradients, and a wave waits for a load only together
     // with everything it requested before it: there the requests go behind the epilogue
@@ -1767,11 +1848,10 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_kc_kernel(const WgradKcP
     if (p.accumulate && !chained) prefetch_next();
     if (!has_next) break;
     cur_u = nxt_u;
-    unit = unit_next;
     par ^= 1;
     ++round;
   }
-  wait_dma<0>();   // the zero loads of the last k-tiles must not land in LDS that a later workgroup owns
+  wait_dma<0>();   // the loads of the last slots must not land in LDS that a later workgroup owns
   if constexpr (DYNAMIC) {
     if (tid == 0) sched_finish(p.sched);
   }
@@ -2337,6 +2417,8 @@ int pk_grouped_swiglu_wgrad_scaled_t(const void* d_out, const void* hsT, const v
   // skewed routing (experts of very different size) needs the dynamic hand-out of units; with a few
   // hundred rows per expert the static one is a few per cent faster
   const bool dynamic = A >= (int64_t)PK_WG_SHORTK_ROWS * E;
+  // the kernels address the gathered operand with 32-bit byte offsets from its base
+  if (((A + row_map_div - 1) / row_map_div) * H * 2 > 0xffffffffll) return PK_ERR_SHAPE;
   auto launch = [&](mf::WgradKcParams& p, bool a_kc) -> int {
     const int64_t units = (int64_t)E * p.nprob * (p.M / 256) * (p.N / 256);
     if (units > 0x7ffffff0ll) return PK_ERR_SHAPE;
@@ -2346,10 +2428,10 @@ int pk_grouped_swiglu_wgrad_scaled_t(const void* d_out, const void* hsT, const v
       if (!p.sched) return PK_ERR_UNSUPPORTED;
     }
     const int id = a_kc ? pk_timing::K_SWIGLU_WGRAD_W13 : pk_timing::K_SWIGLU_WGRAD_W2;
-    if (a_kc && dynamic) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_kc_kernel<256, 256, 32, 2, 4, 4, true, true>), grid, block, 0, s, p);
-    else if (a_kc) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_kc_kernel<256, 256, 32, 2, 4, 4, true, false>), grid, block, 0, s, p);
-    else if (dynamic) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_kc_kernel<256, 256, 32, 4, 2, 4, false, true>), grid, block, 0, s, p);
-    else PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_kc_kernel<256, 256, 32, 4, 2, 4, false, false>), grid, block, 0, s, p);
+    if (a_kc && dynamic) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_pp_kernel<2, 4, true, true>), grid, block, 0, s, p);
+    else if (a_kc) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_pp_kernel<2, 4, true, false>), grid, block, 0, s, p);
+    else if (dynamic) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_pp_kernel<4, 2, false, true>), grid, block, 0, s, p);
+    else PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_pp_kernel<4, 2, false, false>), grid, block, 0, s, p);
     PK_RETURN_IF_LAUNCH_FAILED();
     return PK_OK;
   };

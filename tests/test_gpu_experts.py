@@ -214,10 +214,10 @@ def test_transposed_backward_pair_matches_the_plain_pair(dev, counts, H, I):
     st = starts.cpu().tolist()
     for e, c in enumerate(counts):
         p0 = (st[e] // 64) * 64 + 64 * e
-        c8 = (c + 7) // 8 * 8
+        c32 = (c + 31) // 32 * 32      # zeros up to the end of the expert's last block of 32 rows
         for full, tr in ((d_g, d_gT), (d_u, d_uT), (hs, hsT)):
             # [ldt/32, I, 32] -> [I, ldt]: column i, padded row r
-            blk = tr.permute(1, 0, 2).reshape(I, ldt)[:, p0:p0 + c8]
+            blk = tr.permute(1, 0, 2).reshape(I, ldt)[:, p0:p0 + c32]
             assert torch.equal(blk[:, :c], full[st[e]:st[e] + c].t()), f"expert {e}"
             assert torch.count_nonzero(blk[:, c:]).item() == 0, f"pad columns of expert {e}"
 
