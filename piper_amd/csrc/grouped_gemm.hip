@@ -65,6 +65,12 @@ __device__ __forceinline__ void dma16_s(uint32_t voff, const void* sbase, uint32
                :: "s"(lds_base), "v"(voff), "s"(sbase), "n"(IMM)
                : "memory", "scc");
 }
+// Four bytes per lane straight into LDS (lane l's dword lands at lds_base + 4*l), same address form.
+__device__ __forceinline__ void dma4_s(uint32_t voff, const void* sbase, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2"
+               :: "s"(lds_base), "v"(voff), "s"(sbase)
+               : "memory");
+}
 // f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{}) in order
 template <int I0, int N, typename F>
 __device__ __forceinline__ void static_for_impl(F&& f) {
@@ -658,9 +664,12 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   constexpr int SW = ALIAS ? OUT_COLS : (EPI == EPI_PLAIN && RING + NW * 64 * OUT_COLS > 160 * 1024) ? 32 : OUT_COLS;
   using St = Stage32<SW>;
   constexpr int SMEM_BYTES = ALIAS ? RING : RING + NW * St::BYTES;
-  static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
-  __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
+  // behind it, per wave: the row map entries of the A rows that the wave requests for the next unit
+  constexpr int RM_BYTES = NW * 256;
+  static_assert(SMEM_BYTES + RM_BYTES <= 160 * 1024, "LDS budget");
+  __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES + RM_BYTES];
   constexpr int CPR = BK / 8, RPI = 64 / CPR;            // 16-byte chunks per A row, A rows per dma16
+  static_assert(LA * RPI <= 64, "a wave's A rows of a tile: one entry per lane");
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -737,24 +746,23 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     t.tcol = __builtin_amdgcn_readfirstlane(padded_start(s0, e) + mt * BM);
     t.b_base = uniform_i64(((int64_t)e * p.strideB + (B_KC ? (int64_t)nt * BN_OUT * p.ldb : (int64_t)nt * BN)) * 2);
     t.a_base = p.row_map ? (int64_t)0 : uniform_i64((int64_t)t.row0 * p.lda * 2);
+    if (!p.row_map) {
 #pragma unroll
-    for (int i = 0; i < LA; ++i) {
-      const int rbase = (wave * LA + i) * RPI;     // first tile row of this dma16 (wave-uniform)
-      int src;
-      if (p.row_map) {
-        int sel = 0;
-#pragma unroll
-        for (int r = 0; r < RPI; ++r) {
-          const int rr = min(rbase + r, t.rows - 1);   // rows past the range are never stored
-          const int m = row_map[t.row0 + rr];
-          if (lane / CPR == r) sel = m;
-        }
-        src = fastdiv(sel, p.map_div);
-      } else {
-        src = min(rbase + lane / CPR, t.rows - 1);
+      for (int i = 0; i < LA; ++i) {
+        const int rbase = (wave * LA + i) * RPI;     // first tile row of this dma16 (wave-uniform)
+        t.voff_a[i] = (uint32_t)min(rbase + lane / CPR, t.rows - 1) * row_bytes + a_kofs[i];   // rows past the range are never stored
       }
-      t.voff_a[i] = (uint32_t)src * row_bytes + a_kofs[i];
     }
+  };
+  // With a row map the A rows are gathered: the entries of the wave's LA * RPI tile rows of unit t
+  // go straight into LDS (one 4-byte load per lane, nothing waits for it), and the loader turns
+  // them into lane offsets when it enters the unit, by which time they have landed: every
+  // vector-memory operation of a wave retires in issue order, and the k-loop has by then waited
+  // for tiles requested after them (rows_landed below).
+  int* const rm_area = reinterpret_cast<int*>(smem + SMEM_BYTES) + wave * 64;
+  auto request_rows = [&](const Unit& t) {
+    const int r = wave * (LA * RPI) + lane % (LA * RPI);
+    dma4_s((uint32_t)(t.row0 + min(r, t.rows - 1)) * 4u, p.row_map, lds_addr(rm_area));
   };
 
   // ---- the loader: requests k-tiles in the order the k-loops consume them, NS-1 tiles ahead.
@@ -779,8 +787,14 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   auto ld_take = [&](const Unit& t) {
     ld_a_base = t.a_base;
     ld_b_base = t.b_base;
+    if (p.row_map) {
 #pragma unroll
-    for (int i = 0; i < LA; ++i) ld_voff_a[i] = t.voff_a[i];
+      for (int i = 0; i < LA; ++i)
+        ld_voff_a[i] = (uint32_t)fastdiv(rm_area[i * RPI + lane / CPR], p.map_div) * row_bytes + a_kofs[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < LA; ++i) ld_voff_a[i] = t.voff_a[i];
+    }
     ld_idle = false;
     ld_point(0);
   };
@@ -829,8 +843,17 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   setup(cur_u, unit);
   nxt_u = cur_u;
   int cur = 0;          // ring stage of k-tile 0 of the current unit
+  if (p.row_map) {
+    request_rows(cur_u);
+    wait_dma<0>();
+  }
   ld_take(cur_u);
   issue_prologue(0);
+  // The loader may enter the next unit inside the k-loop only once that unit's row map entries
+  // have landed.  They are requested before the k-loop; the wait at the end of k-tile NS-2 leaves
+  // at most (NS-2)*L younger operations in flight, fewer than were issued after them by then; the
+  // loader enters the next unit during k-tile nkt-NS.
+  const bool rows_landed = !p.row_map || nkt - NS >= NS - 1;
 
   for (;;) {
     int unit_next = -1;
@@ -857,8 +880,14 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     wait_vm_le((NS - 2) * L + st_after);
     block_barrier();
     unit_next = __builtin_amdgcn_readfirstlane(sched_box[par ^ 1]);
-    if (unit_next >= 0) setup(nxt_u, unit_next);
-    next_known = unit_next >= 0;
+    if (unit_next >= 0) {
+      setup(nxt_u, unit_next);
+      if (p.row_map) {
+        request_rows(nxt_u);
+        st_after += 1;      // one more operation younger than this unit's first tiles
+      }
+    }
+    next_known = unit_next >= 0 && rows_landed;
     if constexpr (PP) {
       // Two groups of four waves, one wave of each group on every SIMD, half a k-tile apart: while
       // one group multiplies a k-tile out of registers (16 MFMAs back to back, nothing else), the
@@ -962,6 +991,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
       if (chained) return;
       st_after = 0;
       if (has_next) {
+        if (!rows_landed) wait_dma<0>();     // a k-loop too short to have covered the row map entries
         ld_on_next = true;
         ld_take(nxt_u);
         issue_prologue(cur);
