@@ -366,6 +366,10 @@ int pk_gate_logits(const void* x, int x_dtype, const float* w_gate, const float*
   if (!x || !w_gate || !logits) return PK_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   int sp = gate_fwd_splits(H);
+  // the reduction is split only as far as it takes to give every CU two workgroups: each split
+  // writes and re-reads a [T, E] fp32 partial result, which soon outweighs reading x
+  const int64_t row_tiles = pk_ceil_div(T, 64);
+  while (sp > 1 && row_tiles * (sp / 2) >= 512) sp /= 2;
   if (sp > 1 && (!workspace || workspace_bytes < pk_gate_workspace_bytes(T, H, E))) sp = 1;
   pk_f32mm::Params p = {};
   p.A = x; p.B = w_gate;
