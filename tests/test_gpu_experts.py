@@ -175,6 +175,11 @@ T_CASES = [
     ([700, 0, 0, 2], 512, 256),
     ([256] * 6, 256, 512),
     ([4096, 3000, 1000, 96], 256, 1536),
+    # more weight-gradient tiles than workgroups, so a workgroup walks several units: units handed
+    # out from the counters (long experts) with experts of 0, 1 and 33 rows between long ones ...
+    ([3000, 0, 1, 2500, 33, 0, 700, 600, 500, 400, 300, 64, 32, 70, 100, 96], 1024, 768),
+    # ... and the static hand-out with many short experts (reductions of 0 to 3 k-tiles back to back)
+    ([0, 1, 33, 64, 5, 96, 31, 70, 0, 0, 65, 2] * 24, 256, 256),
 ]
 
 
