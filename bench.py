@@ -79,10 +79,10 @@ def kernel_bytes(cfg) -> dict:
 # them are in the file named here; a kernel without a committed measurement reports null.
 TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.md"
 MEASURED_TRAFFIC_BYTES = {      # (read + written) * 1e6, copied from that file
-    "cfg3": {"swiglu_gate_up": (1060 + 151) * 1e6, "swiglu_down": (484 + 134) * 1e6, "swiglu_dgrad_dh": (801 + 259) * 1e6,
-             "swiglu_dgrad_dx": (975 + 134) * 1e6, "swiglu_wgrad_w13": (343 + 806) * 1e6, "swiglu_wgrad_w2": (207 + 403) * 1e6},
-    "cfg4": {"swiglu_gate_up": (2721 + 605) * 1e6, "swiglu_down": (1292 + 537) * 1e6, "swiglu_dgrad_dh": (2199 + 1020) * 1e6,
-             "swiglu_dgrad_dx": (2601 + 537) * 1e6, "swiglu_wgrad_w13": (1614 + 806) * 1e6, "swiglu_wgrad_w2": (942 + 403) * 1e6},
+    "cfg3": {"swiglu_gate_up": (1070 + 151) * 1e6, "swiglu_down": (483 + 134) * 1e6, "swiglu_dgrad_dh": (807 + 262) * 1e6,
+             "swiglu_dgrad_dx": (976 + 134) * 1e6, "swiglu_wgrad_w13": (355 + 807) * 1e6, "swiglu_wgrad_w2": (213 + 403) * 1e6},
+    "cfg4": {"swiglu_gate_up": (2745 + 606) * 1e6, "swiglu_down": (1292 + 537) * 1e6, "swiglu_dgrad_dh": (2179 + 1023) * 1e6,
+             "swiglu_dgrad_dx": (2612 + 537) * 1e6, "swiglu_wgrad_w13": (1626 + 806) * 1e6, "swiglu_wgrad_w2": (961 + 403) * 1e6},
     "cfg2": {"pack+adamw": (334 + 680 + 2674 + 2378) * 1e6},
 }
 
