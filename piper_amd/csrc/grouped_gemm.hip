@@ -388,12 +388,15 @@ __device__ __forceinline__ int sched_unit_of(unsigned j, int x) {
 // statement, so the compiler never sees a register whose value is still on its way; the wait
 // drains the whole vector-memory counter, so this goes where that counter is about to be
 // drained anyway (after the last store of an epilogue).
-__device__ __forceinline__ unsigned sched_grab(SchedSlot* slot, int x) {
+// The first `base` grab indices of every XCD are not taken from the counter: a workgroup knows its
+// own (its position among the XCD's workgroups, and that plus the XCD's workgroup count where
+// two units are settled at the start), so a kernel starts without a round trip to the counter.
+__device__ __forceinline__ unsigned sched_grab(SchedSlot* slot, int x, unsigned base) {
   unsigned ret;
   const unsigned one = 1u;
   asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)"
                : "=&v"(ret) : "v"(&slot->grabs[x]), "v"(one) : "memory");
-  return ret;
+  return ret + base;
 }
 // Publish a value in LDS for the other waves: the write must have landed before this wave
 // arrives at the next barrier, also on paths that issue no further LDS traffic.
@@ -403,14 +406,14 @@ __device__ __forceinline__ void lds_publish(int* box, int v) {
 }
 // One lane: the next unit for a workgroup of XCD `xcd` (own counter first, then the others), or
 // -1 when all units are taken.  `first` is an already fetched grab index of the own counter.
-__device__ __forceinline__ int sched_resolve(SchedSlot* slot, int xcd, unsigned first, int total) {
+__device__ __forceinline__ int sched_resolve(SchedSlot* slot, int xcd, unsigned first, int total, unsigned base) {
   int unit = sched_unit_of(first, xcd);
   if (unit < total) return unit;
   for (int a = 1; a < NXCD; ++a) {
     const int x = (xcd + a) % NXCD;
     // skip counters that are visibly exhausted (plain read first keeps them from running away)
-    if (sched_unit_of(__atomic_load_n(&slot->grabs[x], __ATOMIC_RELAXED), x) >= total) continue;
-    unit = sched_unit_of(atomicAdd(&slot->grabs[x], 1u), x);
+    if (sched_unit_of(__atomic_load_n(&slot->grabs[x], __ATOMIC_RELAXED) + base, x) >= total) continue;
+    unit = sched_unit_of(atomicAdd(&slot->grabs[x], 1u) + base, x);
     if (unit < total) return unit;
   }
   return -1;
@@ -688,11 +691,8 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   const UnitIndex ui = build_unit_index<BM>(p.starts, p.E, p.n_tiles);
   const int xcd = blockIdx.x % NXCD;
   unsigned grab = 0;                  // lane 0 of wave 0: grab index taken one unit ahead
-  if (tid == 0) {
-    const int first = sched_resolve(p.sched, xcd, sched_grab(p.sched, xcd), ui.total);
-    sched_box[0] = first;
-    if (first >= 0) grab = sched_grab(p.sched, xcd);
-  }
+  const unsigned sched_base = gridDim.x / NXCD;     // grab indices handed out without the counter
+  if (tid == 0) sched_box[0] = sched_resolve(p.sched, xcd, blockIdx.x / NXCD, ui.total, sched_base);
   __syncthreads();
   int unit = __builtin_amdgcn_readfirstlane(sched_box[0]);
   if (unit < 0) {
@@ -849,6 +849,9 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   }
   ld_take(cur_u);
   issue_prologue(0);
+  // the grab index of the second unit: its round trip runs next to the first tiles' (the wait in
+  // it covers both)
+  if (tid == 0) grab = sched_grab(p.sched, xcd, sched_base);
   // The loader may enter the next unit inside the k-loop only once that unit's row map entries
   // have landed.  They are requested before the k-loop; the wait at the end of k-tile NS-2 leaves
   // at most (NS-2)*L younger operations in flight, fewer than were issued after them by then; the
@@ -874,7 +877,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     // unit's addresses (row map lookups included) before the k-loop, which then holds no
     // bookkeeping besides the loader's
     sched_box = reinterpret_cast<int*>(staging_area(cur));
-    if (tid == 0) lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, ui.total));
+    if (tid == 0) lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, ui.total, sched_base));
     // k-tile 0 has landed once only younger operations are in flight: the younger k-tiles and
     // the stores that the previous epilogue issued after its prefetch
     wait_vm_le((NS - 2) * L + st_after);
@@ -982,7 +985,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     const bool has_next = unit_next >= 0;
     // nothing is in flight here, so taking the ticket of the unit after the next one costs
     // one round trip on one wave, not a drain of stores
-    if (has_next && tid == 0) grab = sched_grab(p.sched, xcd);
+    if (has_next && tid == 0) grab = sched_grab(p.sched, xcd, sched_base);
 
     // the next unit's first k-tiles, unless the k-loop has requested them already (then every
     // store of this epilogue is younger than they are)
@@ -1586,13 +1589,13 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_pp_kernel(const WgradKcP
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   };
   unsigned grab = 0;
+  const unsigned sched_base = 2 * G8;      // two units per workgroup are settled without the counters
   int par = 0, round = 0;
   if (tid == 0) {
     int first, second = -1;
     if constexpr (DYNAMIC) {
-      first = sched_resolve(p.sched, xcd, sched_grab(p.sched, xcd), total);
-      if (first >= 0) second = sched_resolve(p.sched, xcd, sched_grab(p.sched, xcd), total);
-      if (second >= 0) grab = sched_grab(p.sched, xcd);
+      first = sched_resolve(p.sched, xcd, blockIdx.x / NXCD, total, sched_base);
+      if (first >= 0) second = sched_resolve(p.sched, xcd, blockIdx.x / NXCD + G8, total, sched_base);
     } else {
       first = unit_at(0);
       if (first >= 0) second = unit_at(1);
@@ -1741,6 +1744,10 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_pp_kernel(const WgradKcP
   ld_enter(cur_u);
   fetch_rows();
   issue_prologue(0);
+  if constexpr (DYNAMIC) {
+    // the grab index of the third unit: its round trip runs next to the first tiles'
+    if (tid == 0 && nx_unit >= 0) grab = sched_grab(p.sched, xcd, sched_base);
+  }
 
   for (;;) {
     next_known = false;
@@ -1831,8 +1838,8 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_pp_kernel(const WgradKcP
     if (has_next && tid == 0) {
       int un2;
       if constexpr (DYNAMIC) {
-        un2 = sched_resolve(p.sched, xcd, grab, total);
-        if (un2 >= 0) grab = sched_grab(p.sched, xcd);
+        un2 = sched_resolve(p.sched, xcd, grab, total, sched_base);
+        if (un2 >= 0) grab = sched_grab(p.sched, xcd, sched_base);
       } else {
         un2 = unit_at(round + 2);
       }
