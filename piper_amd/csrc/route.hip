@@ -308,6 +308,56 @@ __global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ d
   if (threadIdx.x == 0) d_bias[e] = accumulate ? d_bias[e] + s : s;
 }
 
+// The same sum for long inputs in two steps with contiguous reads: block b adds up the rows
+// [b * per, (b+1) * per) of d_logits (256 threads = RP rows x E/4 column groups of 16 bytes, a
+// thread walks every RP-th row with eight rows in flight, the RP partial rows are added in order
+// through LDS), then one thread per column adds the kColsumBlocks partial rows in block order.
+// One block per expert reading a column touches every cache line of d_logits from every XCD.
+constexpr int kColsumBlocks = 64;
+__global__ __launch_bounds__(256) void colsum_partial_kernel(const float* __restrict__ d_logits, int64_t T,
+                                                             int E, float* __restrict__ part) {
+  __shared__ float red[1024];
+  const int cols4 = E / 4, RP = 256 / cols4;
+  const int r = threadIdx.x / cols4, c = threadIdx.x % cols4;
+  const int64_t per = (T + gridDim.x - 1) / gridDim.x;
+  const int64_t t0 = (int64_t)blockIdx.x * per, t1 = t0 + per < T ? t0 + per : T;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (r < RP) {
+    const float4* src = reinterpret_cast<const float4*>(d_logits) + c;
+    int64_t t = t0 + r;
+    for (; t + 7 * RP < t1; t += 8 * RP) {
+      float4 v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = src[(t + i * RP) * cols4];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { acc.x += v[i].x; acc.y += v[i].y; acc.z += v[i].z; acc.w += v[i].w; }
+    }
+    for (; t < t1; t += RP) {
+      const float4 v = src[t * cols4];
+      acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    }
+    reinterpret_cast<float4*>(red)[r * cols4 + c] = acc;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 256) {
+    float s = 0.f;
+    for (int q = 0; q < RP; ++q) s += red[q * E + e];
+    part[(int64_t)blockIdx.x * E + e] = s;
+  }
+}
+__global__ __launch_bounds__(256) void colsum_final_kernel(const float* __restrict__ part, int nblocks, int E,
+                                                           float* __restrict__ d_bias, int accumulate) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= E) return;
+  float v[kColsumBlocks];     // all loads first: one round trip, then the sum in block order
+#pragma unroll
+  for (int b = 0; b < kColsumBlocks; ++b) v[b] = b < nblocks ? part[(int64_t)b * E + e] : 0.f;
+  float s = 0.f;
+#pragma unroll
+  for (int b = 0; b < kColsumBlocks; ++b) s += v[b];
+  d_bias[e] = accumulate ? d_bias[e] + s : s;
+}
+
 // Scratch of pk_sort_by_expert_static: the per-chunk histograms of the counting sort.  Every GPU
 // the library runs on holds its own copy of the array (PK_SORT_STATIC_WORDS * 4 bytes) until the
 // process ends.  In host code the name `scratch` is only a handle for hipGetSymbolAddress: the
@@ -451,9 +501,22 @@ int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const 
     }
   }
   if (d_gate_bias) {
-    PK_LAUNCH_NOCHECK(pk_timing::K_MISC, s, colsum_kernel, dim3((unsigned)E), dim3(256), 0, s, d_logits, T, (int)E,
-                       d_gate_bias, accumulate ? 1 : 0);
-    PK_RETURN_IF_LAUNCH_FAILED();
+    // (the workspace is free again here: the reduction above has consumed the GEMM's partial results)
+    const int64_t part_bytes = (int64_t)kColsumBlocks * E * (int64_t)sizeof(float);
+    if (T >= 32 * kColsumBlocks && E % 4 == 0 && E <= 1024 && workspace && workspace_bytes >= part_bytes &&
+        reinterpret_cast<uintptr_t>(d_logits) % 16 == 0) {
+      float* part = reinterpret_cast<float*>(workspace);
+      PK_LAUNCH_NOCHECK(pk_timing::K_MISC, s, colsum_partial_kernel, dim3(kColsumBlocks), dim3(256), 0, s, d_logits, T,
+                        (int)E, part);
+      PK_RETURN_IF_LAUNCH_FAILED();
+      PK_LAUNCH_NOCHECK(pk_timing::K_MISC, s, colsum_final_kernel, dim3((unsigned)pk_ceil_div(E, 256)), dim3(256), 0, s,
+                        (const float*)part, kColsumBlocks, (int)E, d_gate_bias, accumulate ? 1 : 0);
+      PK_RETURN_IF_LAUNCH_FAILED();
+    } else {
+      PK_LAUNCH_NOCHECK(pk_timing::K_MISC, s, colsum_kernel, dim3((unsigned)E), dim3(256), 0, s, d_logits, T, (int)E,
+                         d_gate_bias, accumulate ? 1 : 0);
+      PK_RETURN_IF_LAUNCH_FAILED();
+    }
   }
   return PK_OK;
 }
