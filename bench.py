@@ -34,6 +34,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bucket", action="store_true")
     ap.add_argument("--no-cfg4", action="store_true", help="skip the cfg4 sub-object of the default run")
+    ap.add_argument("--no-accumulate", action="store_true", help="skip the step that accumulates into existing gradients")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB fp32 device copy (pack_kernel<float,float>) so that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled to a known size")
@@ -87,7 +88,10 @@ MEASURED_TRAFFIC_BYTES = {      # (read + written) * 1e6, copied from that file
 }
 
 
-def bench_region(cfg, steps: int, warmup: int):
+def bench_region(cfg, steps: int, warmup: int, accumulate: bool = False):
+    """accumulate=False: the gradients are cleared before every step (first microbatch of an
+    iteration).  accumulate=True: they are left in place and every step adds to them inside the
+    weight-gradient kernels (any later microbatch; src/executors.py:333-343)."""
     import torch
 
     from piper_amd import _lib, functional as F_
@@ -103,11 +107,15 @@ def bench_region(cfg, steps: int, warmup: int):
     leaves = [t for t in (x, w_gate, bias, w1, w2, w3) if t is not None]
 
     def step():
-        for t in leaves:          # clear_param_grads: first microbatch of an iteration
-            t.grad = None
+        if accumulate:
+            x.grad = None         # the activation gradient is handed on, never accumulated
+        else:
+            for t in leaves:      # clear_param_grads: first microbatch of an iteration
+                t.grad = None
         out = F_.expert_region(x, w_gate, bias, w1, w2, w3, top_k=cfg.top_k, route_norm=cfg.route_norm,
                                route_scale=cfg.route_scale)
-        out.backward(d_out)
+        with F_.accumulate_weight_grads():      # a no-op while the parameters hold no gradient
+            out.backward(d_out)
 
     for _ in range(warmup):
         step()
@@ -220,44 +228,128 @@ def bench_bucket(steps: int, warmup: int):
     }
 
 
+def _median_of_3(fn):
+    """One warm-up pass, then the median of three timed passes (seconds)."""
+    fn()
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return sorted(times)[1]
+
+
+def _host_threads() -> int:
+    import torch
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    return cores
+
+
 def cpu_baseline(cfg):
     """The CPU oracle (un-padded per-expert loop, fp32) on a bounded sample of the same workload:
-    the first tokens of the microbatch with the full set of experts."""
+    the first tokens of the microbatch with the full set of experts.  The fp32 copies of the
+    inputs are made once, outside the timed passes."""
     import torch
 
     from oracle import moe as O
     from piper_amd.configs import make_expert_region_inputs
 
-    cores = os.cpu_count() or 1
-    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-    torch.set_num_threads(cores)
+    cores = _host_threads()
     sample_tokens = min(cfg.tokens, 512)
     inp = make_expert_region_inputs(cfg)
     names = ("x", "w_gate", "w1", "w2", "w3")
+    leaves = {k: (inp[k][:sample_tokens] if k == "x" else inp[k]).float().requires_grad_(True) for k in names}
+    d_out = inp["d_out"][:sample_tokens].float()
+    bias = inp["gate_bias"]
 
     def one():
-        leaves = {k: (inp[k][:sample_tokens] if k == "x" else inp[k]).float().requires_grad_(True) for k in names}
-        bias = inp["gate_bias"]
         out, _ = O.moe_forward(leaves["x"], leaves["w_gate"], bias, leaves["w1"], leaves["w2"], leaves["w3"], cfg.top_k,
                                cfg.route_norm, cfg.route_scale, compute_dtype=torch.float32)
-        torch.autograd.grad(out, list(leaves.values()), inp["d_out"][:sample_tokens].float())
+        torch.autograd.grad(out, list(leaves.values()), d_out)
 
-    one()  # warm-up
-    times = []
-    for _ in range(2):
-        t0 = time.perf_counter()
-        one()
-        times.append(time.perf_counter() - t0)
-    t = sorted(times)[0]
+    t = _median_of_3(one)
     return {"value": sample_tokens / t, "unit": "tokens/s", "cores": cores, "kind": "port",
             "sample": f"first {sample_tokens} of {cfg.tokens} tokens, all {cfg.num_experts} experts, fp32 per-expert loop, "
-                      f"fwd+bwd, best of 2 after 1 warm-up ({t:.2f} s per pass)"}
+                      f"fwd+bwd, median of 3 after 1 warm-up ({t:.2f} s per pass)"}
 
 
-def region_result(cfg, steps: int, warmup: int) -> dict:
+def cpu_baseline_padded_bmm():
+    """The reference's own formulation of the expert segment -- every expert padded to the total
+    row count and run through dense batched matmuls (qwen3_bmm_experts_patch.py:11-50) -- inside the
+    oracle's region, at config 1 (fp32, 256 tokens per microbatch; at config 3 the padded operand
+    alone would take 17 GB).  Beside it the un-padded per-expert loop on the same input."""
+    import torch
+
+    from oracle import moe as O
+    from piper_amd.configs import CFG1, make_expert_region_inputs
+
+    cores = _host_threads()
+    cfg = CFG1
+    inp = make_expert_region_inputs(cfg)
+    names = ("x", "w_gate", "w1", "w2", "w3")
+    leaves = {k: inp[k].float().requires_grad_(True) for k in names}
+    d_out = inp["d_out"].float()
+
+    def region(experts):
+        logits = O.gate_logits(leaves["x"], leaves["w_gate"], None)
+        scores, idx = O.route_topk(logits, cfg.top_k, cfg.route_norm, cfg.route_scale)
+        counts, _starts, perm, _inv = O.sort_by_expert(idx, cfg.num_experts)
+        routed = O.permute(leaves["x"], perm, cfg.top_k)
+        y = experts(leaves["w1"], leaves["w2"], leaves["w3"], routed, counts)
+        out = O.unpermute_combine(y, perm, scores)
+        torch.autograd.grad(out, list(leaves.values()), d_out)
+
+    t_pad = _median_of_3(lambda: region(O.padded_bmm_experts))
+    t_loop = _median_of_3(lambda: region(O.grouped_swiglu))
+    return {"value": cfg.tokens / t_pad, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"config 1 (fp32, one microbatch of {cfg.tokens} tokens, 8 experts top-2), padded batched matmul as in "
+                      f"the reference, fwd+bwd, median of 3 ({t_pad * 1e3:.1f} ms per pass)",
+            "per_expert_loop_tokens_per_s": cfg.tokens / t_loop}
+
+
+def cpu_baseline_bucket():
+    """The reference's bucket arithmetic on the host cores, config 2 at full size: per tensor
+    flat[o:o+n].add_(grad.to(f32)) (src/runtime.py:275-282), then torch.optim.AdamW(foreach=False) on
+    the flat fp32 buffer (the shard optimizer of src/runtime.py:470-473 with the benchmark's
+    optimizer).  Same algorithmic bytes per element as the GPU figure (6 + 28; the CPU side keeps no
+    separate bf16 parameter copy)."""
+    import torch
+
+    from oracle import bucket as OB
+    from piper_amd.configs import ADAMW, bucket_manifest_cfg2
+
+    cores = _host_threads()
+    shapes = [sh for _, sh in bucket_manifest_cfg2()]
+    numels = [math.prod(sh) for sh in shapes]
+    offs, total = OB.plan_offsets(numels, 2, 256)
+    gen = torch.Generator().manual_seed(0)
+    grads = [(torch.randn(sh, generator=gen) * 1e-3).bfloat16() for sh in shapes]
+    flat_g = torch.zeros(total)
+    master = (torch.randn(total, generator=gen) * 0.02).requires_grad_(True)
+    opt = torch.optim.AdamW([master], lr=ADAMW["lr"], betas=ADAMW["betas"], eps=ADAMW["eps"],
+                            weight_decay=ADAMW["weight_decay"], foreach=False)
+
+    def one():
+        flat_g.zero_()
+        OB.pack(flat_g, grads, offs)
+        master.grad = flat_g
+        opt.step()
+
+    t = _median_of_3(one)
+    n = sum(numels)
+    nbytes = 6.0 * n + 28.0 * total
+    return {"value": nbytes / t / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"config 2 at full size ({n} elements in 96 tensors): per-tensor add_ pack + torch.optim.AdamW("
+                      f"foreach=False) on the flat fp32 buffer, median of 3 after 1 warm-up ({t:.2f} s per pass)"}
+
+
+def region_result(cfg, steps: int, warmup: int, accumulate: bool = False) -> dict:
     """Tokens/s, fraction of the bf16 MFMA peak and the roofline of the dominant GEMM kernel for one
     expert-region configuration."""
-    elapsed, kernels = bench_region(cfg, steps, warmup)
+    elapsed, kernels = bench_region(cfg, steps, warmup, accumulate)
     host_enqueue = kernels.pop("__host_enqueue_s")
     dominant = kernels.pop("__dominant")
     ms_per_step = elapsed / steps * 1e3
@@ -342,10 +434,20 @@ def main():
         c4 = region_result(CFG4, args.steps, args.warmup)
         result["cfg4"] = {k: c4[k] for k in ("value", "unit", "ms_per_step", "config", "mfma_frac_of_peak_region",
                                              "gemm_tflops_region", "roofline", "kernels_ms_per_step", "gemm_kernels_tflops")}
+    if not args.no_accumulate:
+        # the same step on a later microbatch of an iteration: the parameter gradients exist and the
+        # weight-gradient kernels add to them (one more read of 3 x E x I x H gradients per step)
+        acc = region_result(cfg, args.steps, args.warmup, accumulate=True)
+        result["accumulate"] = {k: acc[k] for k in ("value", "unit", "ms_per_step", "mfma_frac_of_peak_region",
+                                                    "gemm_tflops_region", "kernels_ms_per_step")}
+        result["accumulate"]["vs_clearing_step"] = acc["ms_per_step"] / result["ms_per_step"]
     if not args.no_bucket:
         result["bucket"] = bench_bucket(max(5, args.steps), max(2, args.warmup))
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg)
+        result["cpu_baseline"]["padded_bmm_cfg1"] = cpu_baseline_padded_bmm()
+        if not args.no_bucket:
+            result["bucket"]["cpu_baseline"] = cpu_baseline_bucket()
     print(json.dumps(result))
 
 

@@ -49,6 +49,15 @@ typedef void* pk_stream_t;
 PK_API int pk_version(void);
 PK_API const char* pk_status_string(int status);
 
+/* Optional set-up for the CURRENT device: resolves the device addresses of the library's own
+ * device arrays (the scheduling counters of the grouped GEMMs, the scratch of
+ * pk_sort_by_expert_static) and reads the device's CU count.  Every entry point does this by
+ * itself on its first call on a device; a caller that records launches into a HIP graph calls
+ * pk_init() (or makes one ordinary call of each entry point it will record) on that device BEFORE
+ * the capture starts, because symbol look-ups are not legal while a stream is capturing.
+ * No counterpart in the reference (its operators are ATen calls). */
+PK_API int pk_init(void);
+
 /* ------------------------------------------------------------------ routing */
 
 /* logits[T,E] (f32) = x[T,H] (x_dtype) . w_gate[E,H]^T (f32) + gate_bias[E] (f32, may be NULL),
@@ -280,7 +289,13 @@ PK_API int pk_grouped_swiglu_wgrad_scaled(const void* d_out, const void* hs, con
  * 0 when the shape or dtype has no such path (use the entry points above then).
  * pk_grouped_swiglu_wgrad_scaled_t computes the same d_w1, d_w2, d_w3 as
  * pk_grouped_swiglu_wgrad_scaled from d_out, x (through row_map / row_map_div) and the transposed
- * copies.  Both replace the autograd of qwen3_bmm_experts_patch.py:39-41 like the pair above. */
+ * copies.  Both replace the autograd of qwen3_bmm_experts_patch.py:39-41 like the pair above.
+ * Restriction of pk_grouped_swiglu_wgrad_scaled_t: the last 32-row block of an expert multiplies
+ * the zeros of the transposed copy with the rows of x / d_out that the row map names behind the
+ * expert's last row (rows of the next expert's tokens).  Zero times a finite value is zero; zero
+ * times Inf or NaN is NaN.  A non-finite row of x or d_out can therefore reach the weight gradients
+ * of the expert in front of the one it was routed to, which pk_grouped_swiglu_wgrad_scaled (rows
+ * past an expert's end read as zeros) confines to its own experts. */
 PK_API int64_t pk_grouped_swiglu_transposed_ld(int64_t A, int64_t H, int64_t I, int64_t E, int dtype);
 PK_API int pk_grouped_swiglu_dgrad_dh_scaled_t(const void* d_out, const int32_t* row_map, int64_t row_map_div,
                                         const float* scores, const void* w2, const void* g,
@@ -293,6 +308,18 @@ PK_API int pk_grouped_swiglu_wgrad_scaled_t(const void* d_out, const void* hsT, 
                                      const int32_t* starts, const int32_t* expert_order, void* d_w1,
                                      void* d_w2, void* d_w3, int accumulate, int64_t A, int64_t H,
                                      int64_t I, int64_t E, int dtype, pk_stream_t stream);
+
+/* Diagnostic, HOST only (touches no device): index of the set of scheduling counters that the
+ * persistent grouped GEMMs use for launches with this key.  The library keeps PK_SCHED_SETS sets per
+ * device and gives every (stream, capture sequence) pair a set of its own, so that launches that can
+ * overlap never share counters: launches on one stream are ordered, and launches recorded into a
+ * HIP graph (capture_sequence != 0: 1 + the id hipStreamGetCaptureInfo reports) keep the set of
+ * their capture for the life of the graph.  thread_key is 0 except for hipStreamPerThread, which
+ * names a different stream in every host thread.  With more than PK_SCHED_SETS keys on a device the
+ * sets are shared round-robin, and two launches that share one must not overlap.  No counterpart
+ * in the reference. */
+#define PK_SCHED_SETS 1024
+PK_API int pk_sched_slot_index(int device, uint64_t stream_handle, uint64_t capture_sequence, uint64_t thread_key);
 
 /* ------------------------------------------------------------- ZeRO bucket path */
 

@@ -26,6 +26,8 @@ _p = C.c_void_p
 SIGNATURES = {
     "pk_version": (_c_int, []),
     "pk_status_string": (C.c_char_p, [_c_int]),
+    "pk_init": (_c_int, []),
+    "pk_sched_slot_index": (_c_int, [_c_int, C.c_uint64, C.c_uint64, C.c_uint64]),
     "pk_gate_workspace_bytes": (_c_i64, [_c_i64, _c_i64, _c_i64]),
     "pk_gate_logits": (_c_int, [_p, _c_int, _p, _p, _p, _c_i64, _c_i64, _c_i64, _p, _c_i64, _p]),
     "pk_route_topk": (_c_int, [_p, _c_i64, _c_i64, _c_i64, _c_int, _c_f32, _p, _p, _p]),
@@ -105,6 +107,21 @@ def status_string(status: int) -> str:
     return load().pk_status_string(int(status)).decode()
 
 
+_ready_devices: set = set()
+
+
+def init_device() -> None:
+    """pk_init() once per device: the library's device arrays are resolved before any launch, so
+    that the first launch of an entry point may already sit inside a HIP graph capture."""
+    dev = torch.cuda.current_device()
+    if dev in _ready_devices:
+        return
+    rc = load().pk_init()
+    if rc != 0:
+        raise RuntimeError(f"pk_init failed with status {rc}: {status_string(rc)}")
+    _ready_devices.add(dev)
+
+
 def call(name: str, *args):
     """Call an int-returning entry point and raise RuntimeError on a non-zero status."""
     rc = getattr(load(), name)(*args)
@@ -164,6 +181,7 @@ def ptr(t: torch.Tensor | None):
 def current_stream(device: torch.device | None = None):
     """The hipStream_t of torch's current stream, so kernels respect `torch.cuda.stream(...)`
     exactly like the ATen ops they replace (src/executors.py:231-232)."""
+    init_device()
     return torch.cuda.current_stream(device).cuda_stream
 
 

@@ -46,6 +46,15 @@ class BucketState:
     param_shard_info: tuple | None = None            # (shard_start, shard_size, orig_numel)
     param_view_specs: list = field(default_factory=list)  # (param, offset, numel, shape)
     full_params_fresh: bool = False
+    # Flat buffers for the parameters of this compute bucket that have another dtype than
+    # flat_params (the fp32 router gate of a bf16 layer): BucketStates without a forward_fn that
+    # ParamStorage zeroes, packs, unflattens and steps together with this one.  The reference has
+    # no such field: its flatten concatenates the parameters of a bucket whatever their dtype
+    # (src/actor.py:534).
+    companions: list = field(default_factory=list)
+
+    def with_companions(self) -> list:
+        return [self] + list(self.companions)
 
     def weights(self) -> list:
         return [self.forward_args[i] for i in self.param_idxs if self.forward_args[i] is not None]
@@ -133,12 +142,15 @@ class RuntimeState:
 
 class _DeferredFree:
     """A release that has to wait for a GPU event (src/runtime.py:284-310).  The reference hands
-    `evt.synchronize(); free()` to a one-thread pool and keeps the Future; here the wait and the
-    release run when somebody asks for the result, which is what every consumer of the Future does
-    before it touches the buffer again (`wait_pending_free`, `drain_pending_frees`)."""
+    `evt.synchronize(); free()` to a one-thread pool and keeps the Future; here the release runs
+    when somebody asks for the result, which is what every consumer of the Future does before it
+    touches the buffer again (`wait_pending_free`, `drain_pending_frees`).  The host waits for the
+    event only when the release returns memory (`frees_memory`): with a data-parallel group of one
+    nothing is returned -- the bucket is only marked stale -- and blocking the host there would stop
+    it from queueing work ahead of the GPU for no benefit."""
 
-    def __init__(self, evt, release):
-        self._evt, self._release, self._done = evt, release, False
+    def __init__(self, evt, release, frees_memory: bool = True):
+        self._evt, self._release, self._frees_memory, self._done = evt, release, frees_memory, False
 
     def done(self) -> bool:
         return self._done or self._evt is None or self._evt.query()
@@ -146,7 +158,7 @@ class _DeferredFree:
     def result(self) -> None:
         if self._done:
             return
-        if self._evt is not None:
+        if self._evt is not None and self._frees_memory:
             self._evt.synchronize()
         self._release()
         self._done = True
@@ -194,7 +206,7 @@ class ParamStorage:
         if ubid is None or ubid not in self.stages.param_sharded_ubids:
             return
         self.wait_pending_free(self.pending_param_frees, ubid)
-        self.pending_param_frees[ubid] = _DeferredFree(evt, lambda: self.free_full_params(ubid))
+        self.pending_param_frees[ubid] = _DeferredFree(evt, lambda: self.free_full_params(ubid), frees_memory=False)
 
     def defer_free_full_grads(self, ubid, evt) -> None:
         if ubid is None or ubid not in self.stages.grad_sharded_ubids:
@@ -203,17 +215,21 @@ class ParamStorage:
         # the pack that recorded `evt` has already dropped the per-tensor gradients, and with a
         # data-parallel group of one the flat buffer is also the optimizer's shard gradient: after the
         # event nothing is left to release (a late `free_full_grads` would only wipe newer gradients)
-        self.pending_grad_frees[ubid] = _DeferredFree(evt, lambda: None)
+        self.pending_grad_frees[ubid] = _DeferredFree(evt, lambda: None, frees_memory=False)
+
+    def _all_states(self):
+        for bucket in self.stages.buckets.values():
+            yield from bucket.with_companions()
 
     def clear_param_grads(self) -> None:
-        for bucket in self.stages.buckets.values():
+        for bucket in self._all_states():
             for p, *_ in bucket.param_view_specs:
                 p.grad = None
 
     def zero_grad_buffers(self, stream: torch.cuda.Stream | None = None) -> None:
         """src/runtime.py:223-229."""
         with torch.cuda.stream(stream):
-            for bucket in self.stages.buckets.values():
+            for bucket in self._all_states():
                 if bucket.flat_grads is not None:
                     ops.bucket_zero(bucket.flat_grads)
                 rs = bucket.reduce_scatter_grads
@@ -227,7 +243,10 @@ class ParamStorage:
             return
         if ubid in self.stages.grad_sharded_ubids:
             self.wait_pending_free(self.pending_grad_frees, ubid)
-        bucket = self.stages.bucket(ubid)
+        for bucket in self.stages.bucket(ubid).with_companions():
+            self._pack_one(bucket, stream)
+
+    def _pack_one(self, bucket: BucketState, stream) -> None:
         specs = bucket.param_view_specs
         if not specs:
             return
@@ -254,21 +273,22 @@ class ParamStorage:
 
     def alloc_full_params(self, ubid) -> None:
         """Unflatten (src/runtime.py:312-352): make every parameter a view of the flat bucket."""
-        bucket = self.stages.bucket(ubid)
         self.wait_pending_free(self.pending_param_frees, ubid)
-        full = bucket.flat_params
-        assert full is not None, f"alloc_full_params: missing flat_params buffer for ubid={ubid}"
-        assert bucket.param_view_specs, f"alloc_full_params: missing param_view_specs for ubid={ubid}"
-        for param, offset, numel, shape in bucket.param_view_specs:
-            if param.data_ptr() != full.data_ptr() + offset * full.element_size():
-                param.data = full[offset:offset + numel].view(shape)
-            param.requires_grad_(True)
-        bucket.full_params_fresh = True
+        for bucket in self.stages.bucket(ubid).with_companions():
+            full = bucket.flat_params
+            assert full is not None, f"alloc_full_params: missing flat_params buffer for ubid={ubid}"
+            assert bucket.param_view_specs, f"alloc_full_params: missing param_view_specs for ubid={ubid}"
+            for param, offset, numel, shape in bucket.param_view_specs:
+                if param.data_ptr() != full.data_ptr() + offset * full.element_size():
+                    param.data = full[offset:offset + numel].view(shape)
+                param.requires_grad_(True)
+            bucket.full_params_fresh = True
 
     def free_full_params(self, ubid) -> None:
         """One device keeps the only copy of the parameters, so there is nothing to release;
         the bucket is only marked stale (src/runtime.py:354-371)."""
-        self.stages.bucket(ubid).full_params_fresh = False
+        for bucket in self.stages.bucket(ubid).with_companions():
+            bucket.full_params_fresh = False
 
     def alloc_full_grads(self, ubid, stream: torch.cuda.Stream | None = None) -> None:
         bucket = self.stages.bucket(ubid)
@@ -280,9 +300,9 @@ class ParamStorage:
                 bucket.reduce_scatter_grads = bucket.flat_grads
 
     def free_full_grads(self, ubid) -> None:
-        bucket = self.stages.bucket(ubid)
-        for param, *_ in bucket.param_view_specs:
-            param.grad = None
+        for bucket in self.stages.bucket(ubid).with_companions():
+            for param, *_ in bucket.param_view_specs:
+                param.grad = None
 
     def all_gather_full_params(self, ubid, stream: torch.cuda.Stream | None = None) -> int:
         """dp_degree == 1: the shard is the whole bucket, so the gather moves no bytes."""
@@ -290,7 +310,7 @@ class ParamStorage:
         return 0
 
     def has_zero_shard_optimizers(self) -> bool:
-        return any(b.shard_optimizer is not None for b in self.stages.buckets.values())
+        return any(b.shard_optimizer is not None for b in self._all_states())
 
     def step_zero_shard_optimizers(self, stream: torch.cuda.Stream | None = None,
                                    reduce_scatter_events: dict | None = None) -> None:
@@ -299,7 +319,7 @@ class ParamStorage:
         if stream is not None:
             for evt in (reduce_scatter_events or {}).values():
                 stream.wait_event(evt)
-        for bucket in self.stages.buckets.values():
+        for bucket in self._all_states():
             opt = bucket.shard_optimizer
             if opt is None or bucket.reduce_scatter_grads is None:
                 continue

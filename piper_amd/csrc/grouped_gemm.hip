@@ -1,16 +1,22 @@
 // Grouped SwiGLU expert GEMMs (forward, input gradient, weight gradient).
 //   bf16: v_mfma_f32_32x32x16_bf16 tiles fed by a ring of direct-to-LDS loads.
-//         Forward and input gradient: persistent workgroups (one per CU) that take
-//         (expert, row tile, column tile) units from per-XCD counters, 256x256x32 block tiles
-//         with 8 waves, fused SwiGLU / SwiGLU-backward epilogues, permute fused into the
-//         A-operand loader; ragged row tiles are located on the device from starts[] (no host
-//         sync).  Weight gradient: one workgroup per (expert, output tile), 256x256x64 tiles.
+//         Forward and input gradient (ragged_m_kernel): persistent workgroups (one per CU) that
+//         take (expert, row tile, column tile) units from per-XCD counters, 256x256x32 or
+//         128x256x64 block tiles with 8 waves, fused SwiGLU / SwiGLU-backward epilogues, permute
+//         fused into the A-operand loader; ragged row tiles are located on the device from
+//         starts[] (no host sync).  Weight gradient: wgrad_pp_kernel (persistent, 256x256x32, one
+//         operand from the transposed copies the scaled SwiGLU backward writes) for the fused
+//         region; wgrad_kernel (one workgroup per (expert, output tile), both operands through the
+//         transposing LDS read) for the piecewise entry points.
 //   f32 : tiled FMA kernel (simt_gemm.h) + elementwise SwiGLU kernels; exact fp32 arithmetic.
 #include "pk_common.h"
 #include "simt_gemm.h"
-#include <atomic>
+#include <functional>
 #include <initializer_list>
+#include <map>
 #include <mutex>
+#include <thread>
+#include <tuple>
 #include <type_traits>
 
 namespace {
@@ -369,11 +375,12 @@ __device__ __forceinline__ void locate_unit(const UnitIndex& ui, const_i32_ptr s
 // consecutive units; chunk c belongs to XCD c % 8, whose workgroups take its units one at a
 // time from a counter, so the workgroups of an XCD always run neighbouring units (shared
 // operands stay in that XCD's L2) while uneven unit costs still balance.  A workgroup whose own
-// XCD has run dry takes units from the other XCDs' counters.  Every launch uses one slot of a
-// pool of counter sets; the last workgroup to finish zeroes the slot again, so no memset
-// precedes a launch and launches in flight on different streams do not share counters.
+// XCD has run dry takes units from the other XCDs' counters.  Every launch uses one set of a
+// pool of counter sets, chosen by its stream (sched_slot_for_launch); the last workgroup to finish
+// zeroes the set again, so no memset precedes a launch and launches in flight on different
+// streams do not share counters.
 constexpr int SCHED_CHUNK = 32;
-constexpr int SCHED_SLOTS = 1024;
+constexpr int SCHED_SLOTS = PK_SCHED_SETS;
 struct SchedSlot {
   unsigned grabs[NXCD];
   unsigned finished;
@@ -669,8 +676,12 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   constexpr int SMEM_BYTES = ALIAS ? RING : RING + NW * St::BYTES;
   // behind it, per wave: the row map entries of the A rows that the wave requests for the next unit
   constexpr int RM_BYTES = NW * 256;
-  static_assert(SMEM_BYTES + RM_BYTES <= 160 * 1024, "LDS budget");
-  __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES + RM_BYTES];
+  // and the two words through which one lane hands the next unit's index to the workgroup.  They
+  // have a place of their own: inside the ring they would sit in a stage that the first memory
+  // phase of the next k-loop may already be filling while a late wave still reads them.
+  constexpr int BOX_BYTES = 16;
+  static_assert(SMEM_BYTES + RM_BYTES + BOX_BYTES <= 160 * 1024, "LDS budget");
+  __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES + RM_BYTES + BOX_BYTES];
   constexpr int CPR = BK / 8, RPI = 64 / CPR;            // 16-byte chunks per A row, A rows per dma16
   static_assert(LA * RPI <= 64, "a wave's A rows of a tile: one entry per lane");
 
@@ -685,9 +696,8 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   const const_i32_ptr row_map = as_const(p.row_map);
 
   // ---- first unit of this workgroup
-  // the next unit, written by one lane, double buffered; it lives in the first bytes of the
-  // staging area, which is idle between the first two barriers of a k-loop (nkt >= 2)
-  int* sched_box = reinterpret_cast<int*>(staging_area(0));
+  // the next unit, written by one lane, double buffered
+  int* const sched_box = reinterpret_cast<int*>(smem + SMEM_BYTES + RM_BYTES);
   const UnitIndex ui = build_unit_index<BM>(p.starts, p.E, p.n_tiles);
   const int xcd = blockIdx.x % NXCD;
   unsigned grab = 0;                  // lane 0 of wave 0: grab index taken one unit ahead
@@ -876,7 +886,6 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     // unit and leaves it in LDS; everyone reads it behind the barrier below and resolves the
     // unit's addresses (row map lookups included) before the k-loop, which then holds no
     // bookkeeping besides the loader's
-    sched_box = reinterpret_cast<int*>(staging_area(cur));
     if (tid == 0) lds_publish(&sched_box[par ^ 1], sched_resolve(p.sched, xcd, grab, ui.total, sched_base));
     // k-tile 0 has landed once only younger operations are in flight: the younger k-tiles and
     // the stores that the previous epilogue issued after its prefetch
@@ -1911,23 +1920,71 @@ inline int persistent_grid() {
   return cached;
 }
 
-// Counter set for one launch on the current device (nullptr if the pool cannot be resolved).
-inline SchedSlot* sched_slot_for_launch() {
-  constexpr int MAX_DEV = 64;
-  static SchedSlot* base[MAX_DEV] = {};
-  static std::mutex mu;
-  static std::atomic<unsigned> seq{0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) return nullptr;
-  if (!base[dev]) {
-    std::lock_guard<std::mutex> lock(mu);
-    if (!base[dev]) {
-      void* ptr = nullptr;
-      if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_sched_pool)) != hipSuccess || !ptr) return nullptr;
-      base[dev] = (SchedSlot*)ptr;
-    }
+// Which counter set a launch uses.  Launches on one stream run one after the other and every
+// launch leaves its set zeroed, so ONE set per stream is enough, and two launches share a set only
+// if they cannot overlap.  The key of a set is (stream, capture sequence): a launch recorded into
+// a HIP graph keeps its set for the life of the graph, which may replay next to eager work on the
+// stream it was captured on, so a capture gets sets of its own (per stream of the capture: the
+// streams of a forked capture run side by side inside the graph).  hipStreamPerThread is one
+// handle for a different stream in every host thread, so there the thread is part of the key.
+// When more keys than sets have been seen, sets are shared round-robin.
+struct SchedKey {
+  const void* stream;
+  unsigned long long capture;
+  size_t thread;
+  bool operator<(const SchedKey& o) const {
+    return std::tie(stream, capture, thread) < std::tie(o.stream, o.capture, o.thread);
   }
-  return base[dev] + (seq.fetch_add(1) % SCHED_SLOTS);
+};
+struct SchedDirectory {
+  std::mutex mu;
+  std::map<SchedKey, int> slot_of[PK_MAX_DEVICES];
+  int next[PK_MAX_DEVICES] = {};
+  SchedSlot* base[PK_MAX_DEVICES] = {};
+};
+SchedDirectory& sched_directory() {
+  static SchedDirectory d;
+  return d;
+}
+// Index of the set for a key on device `dev` (assigns the next set to a key seen for the first time).
+int sched_slot_index(int dev, const void* stream, unsigned long long capture, size_t thread) {
+  SchedDirectory& d = sched_directory();
+  std::lock_guard<std::mutex> lock(d.mu);
+  const SchedKey key{stream, capture, thread};
+  auto it = d.slot_of[dev].find(key);
+  if (it != d.slot_of[dev].end()) return it->second;
+  const int slot = d.next[dev]++ % SCHED_SLOTS;
+  d.slot_of[dev].emplace(key, slot);
+  return slot;
+}
+// Device address of the pool on the current device, looked up once per device.
+SchedSlot* sched_pool_base(int dev) {
+  SchedDirectory& d = sched_directory();
+  std::lock_guard<std::mutex> lock(d.mu);
+  if (!d.base[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_sched_pool)) != hipSuccess || !ptr) return nullptr;
+    d.base[dev] = (SchedSlot*)ptr;
+  }
+  return d.base[dev];
+}
+// Counter set for one launch on stream `s` of the current device (nullptr if the pool cannot be
+// resolved).
+inline SchedSlot* sched_slot_for_launch(hipStream_t s) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= PK_MAX_DEVICES) return nullptr;
+  SchedSlot* const base = sched_pool_base(dev);
+  if (!base) return nullptr;
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  unsigned long long capture = 0;
+  if (hipStreamGetCaptureInfo(s, &status, &capture) != hipSuccess) {
+    (void)hipGetLastError();
+    status = hipStreamCaptureStatusNone;
+  }
+  if (status != hipStreamCaptureStatusActive) capture = 0;
+  else capture += 1;      // 0 stands for "not capturing"
+  const size_t thread = s == hipStreamPerThread ? std::hash<std::thread::id>{}(std::this_thread::get_id()) : 0;
+  return base + sched_slot_index(dev, (const void*)s, capture, thread);
 }
 
 template <int BM, int BN, int BK, int WMW, int WNW, int NS, bool B_KC, int EPI>
@@ -1940,7 +1997,7 @@ int launch_ragged_m(RaggedMParams p, int64_t A_rows, int kernel_id, hipStream_t 
   if (p.lda * 2 > 0x7fffffffll || (a_span_rows + 1) * p.lda * 2 > 0xffffffffll) return PK_ERR_SHAPE;
   if ((int64_t)p.Kseg * p.nseg < 2 * BK) return PK_ERR_SHAPE;
   const int64_t grid = max_units < persistent_grid() ? round_up_xcd(max_units) : persistent_grid();
-  p.sched = sched_slot_for_launch();
+  p.sched = sched_slot_for_launch(s);
   if (!p.sched) return PK_ERR_UNSUPPORTED;
   PK_LAUNCH_NOCHECK(kernel_id, s, (ragged_m_kernel<BM, BN, BK, WMW, WNW, NS, B_KC, EPI>),
                     dim3((unsigned)grid), dim3(64 * WMW * WNW), 0, s, p);
@@ -2063,9 +2120,10 @@ int simt_ragged_k(const void* A, int64_t lda, const int32_t* a_map, const void* 
 #define PK_RM_SHORT_ROWS 512
 // Output widths that are a multiple of 128 but not of 256.
 #define PK_RM_ALT 128, 128, 64, 2, 2, 4
-// Weight gradient: 256x256x64 in a 2-stage ring; with fewer than PK_WG_SHORTK_ROWS rows per expert on
-// average 32-deep tiles in a 4-stage ring with the loads spread between the MFMAs (measured
-// against the 64-deep ring: -1.8 % at 256 rows per expert, +7 % at 1,024).
+// Weight gradient of the piecewise entry points (wgrad_kernel; the fused region runs
+// wgrad_pp_kernel, whose tile is fixed): 256x256x64 in a 2-stage ring; with fewer than
+// PK_WG_SHORTK_ROWS rows per expert on average 32-deep tiles in a 4-stage ring with the loads spread
+// between the MFMAs (measured against the 64-deep ring: -1.8 % at 256 rows per expert, +7 % at 1,024).
 #define PK_WG_BIG 256, 256, 64, 2, 4, 2
 #define PK_WG_BIG_THREADS 512
 #define PK_WG_BIG_SHORTK 256, 256, 32, 2, 4, 4
@@ -2142,7 +2200,22 @@ int wgrad_simt(const void* dy, const int32_t* dy_map, const void* h, const void*
 
 }  // namespace
 
+// Resolves, for the current device, what the grouped GEMMs otherwise look up on their first launch.
+int pk_init_grouped_gemm() {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= PK_MAX_DEVICES) return PK_ERR_UNSUPPORTED;
+  (void)mf::persistent_grid();
+  return mf::sched_pool_base(dev) ? PK_OK : PK_ERR_UNSUPPORTED;
+}
+
 extern "C" {
+
+int pk_sched_slot_index(int device, uint64_t stream_handle, uint64_t capture_sequence, uint64_t thread_key) {
+  if (device < 0 || device >= PK_MAX_DEVICES) return PK_ERR_ARG;
+  return mf::sched_slot_index(device, (const void*)(uintptr_t)stream_handle, capture_sequence, (size_t)thread_key);
+}
 
 int pk_grouped_swiglu_fwd(const void* x_rows, const int32_t* row_map, int64_t row_map_div,
                           const void* w1, const void* w2, const void* w3,
@@ -2461,7 +2534,7 @@ int pk_grouped_swiglu_wgrad_scaled_t(const void* d_out, const void* hsT, const v
     if (units > 0x7ffffff0ll) return PK_ERR_SHAPE;
     const dim3 grid((unsigned)(units < mf::persistent_grid() ? mf::round_up_xcd(units) : mf::persistent_grid())), block(512);
     if (dynamic) {
-      p.sched = mf::sched_slot_for_launch();
+      p.sched = mf::sched_slot_for_launch(s);
       if (!p.sched) return PK_ERR_UNSUPPORTED;
     }
     const int id = a_kc ? pk_timing::K_SWIGLU_WGRAD_W13 : pk_timing::K_SWIGLU_WGRAD_W2;

@@ -13,6 +13,10 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 #define PK_WAVE 64
+#define PK_MAX_DEVICES 64
+
+// Per-source set-up behind pk_init (current device).
+int pk_init_grouped_gemm();
 
 #define PK_RETURN_IF_LAUNCH_FAILED()        \
   do {                                      \

@@ -365,7 +365,7 @@ __global__ __launch_bounds__(256) void colsum_final_kernel(const float* __restri
 static __device__ __align__(256) int32_t scratch[PK_SORT_STATIC_WORDS];
 
 int32_t* sort_scratch_for_current_device() {
-  constexpr int MAX_DEV = 64;
+  constexpr int MAX_DEV = PK_MAX_DEVICES;
   static int32_t* ptr[MAX_DEV] = {};
   static std::mutex mu;
   int dev = 0;
@@ -384,6 +384,11 @@ int32_t* sort_scratch_for_current_device() {
 extern "C" {
 
 int pk_version(void) { return 100; }
+
+int pk_init(void) {
+  if (!sort_scratch_for_current_device()) return PK_ERR_UNSUPPORTED;
+  return pk_init_grouped_gemm();
+}
 
 const char* pk_status_string(int status) {
   switch (status) {

@@ -94,7 +94,9 @@ class ComputeExecutor:
             if not roots:
                 raise AssertionError(f"backward of bucket {ubid!r}, microbatch {mb_idx}: no output of the "
                                      "bucket received a gradient from its consumer")
-        with torch.cuda.stream(compute_stream):
+        # the backward accumulates into .grad; the HIP operators add to gradients that exist
+        # already (later microbatches of an iteration) inside their kernels
+        with torch.cuda.stream(compute_stream), F_.accumulate_weight_grads():
             torch.autograd.backward(roots, grads)
         received = [t.grad for t in (inp_with_grad or ()) if t.grad is not None]
         return {"send_output": received} if received else None

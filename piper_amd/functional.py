@@ -48,23 +48,28 @@ def _sorted_tables(top_idx: torch.Tensor, num_experts: int):
     """(counts, starts, perm, inv_perm) of the counting sort of `top_idx`, computed once per routing
     result: the tables ride on the index tensor, and the inverse permutation rides on `perm`, so the
     piecewise operators that follow (reorder, permute backward, combine) launch no second sort."""
+    # valid for this tensor object, these contents (autograd's version counter moves with every
+    # in-place write) and this expert count; a view or a clone is another object and is sorted again
+    key = (top_idx._version, int(num_experts))
     cached = getattr(top_idx, "_pk_sorted", None)
-    if cached is None or cached[0].numel() != num_experts:
-        cached = ops.sort_by_expert(top_idx, num_experts)
-        cached[2]._pk_inverse = cached[3]
+    if cached is None or cached[0] != key:
+        tables = ops.sort_by_expert(top_idx, num_experts)
+        tables[2]._pk_inverse = (tables[2]._version, tables[3])
+        cached = (key, tables)
         top_idx._pk_sorted = cached
-    return cached
+    return cached[1]
 
 
 def _inverse_of(perm: torch.Tensor) -> torch.Tensor:
     """inv_perm for a permutation produced by `reorder` (cached there); any other permutation is
     inverted once and remembered on the tensor."""
-    inv = getattr(perm, "_pk_inverse", None)
-    if inv is None:
+    cached = getattr(perm, "_pk_inverse", None)
+    if cached is None or cached[0] != perm._version:
         inv = torch.empty_like(perm)
         inv[perm.long()] = torch.arange(perm.numel(), dtype=perm.dtype, device=perm.device)
-        perm._pk_inverse = inv
-    return inv
+        cached = (perm._version, inv)
+        perm._pk_inverse = cached
+    return cached[1]
 
 
 def router(x, w_gate, gate_bias=None, *, top_k: int, route_norm: bool, route_scale: float = 1.0):
@@ -88,12 +93,13 @@ class _PermuteFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, perm, top_k):
         ctx.top_k = top_k
-        ctx.inv_perm = _inverse_of(perm)
+        ctx.save_for_backward(_inverse_of(perm))
         return ops.permute_fwd(x, perm, top_k)
 
     @staticmethod
     def backward(ctx, d_routed):
-        return ops.permute_bwd(d_routed, ctx.inv_perm, ctx.top_k), None, None
+        (inv_perm,) = ctx.saved_tensors
+        return ops.permute_bwd(d_routed, inv_perm, ctx.top_k), None, None
 
 
 def permute(x: torch.Tensor, token_indices_experts_sorted: torch.Tensor, top_k: int) -> torch.Tensor:
@@ -121,6 +127,11 @@ class _BmmExpertsFn(torch.autograd.Function):
         d_w1 = d_w2 = d_w3 = None
         if all(ctx.needs_input_grad[:3]) and _can_defer(*ctx.params):
             _queue_expert_wgrad(ctx.params, d_y, h, d_g, d_u, x, starts, None, 1, None)
+        elif (_ACCUMULATE_INTO_GRAD and all(ctx.needs_input_grad[:3])
+              and all(_accumulates_in_place(p) for p in ctx.params)):
+            p1, p2, p3 = ctx.params
+            ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, w1.shape[0], d_w1=p1.grad, d_w2=p2.grad, d_w3=p3.grad,
+                                     accumulate=True)
         elif any(ctx.needs_input_grad[:3]):
             d_w1, d_w2, d_w3 = ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, w1.shape[0])
         return d_w1, d_w2, d_w3, d_x, None
@@ -277,6 +288,61 @@ class defer_weight_grads:
         _WGRAD_QUEUE = self._prev
 
 
+_ACCUMULATE_INTO_GRAD = False
+
+
+class accumulate_weight_grads:
+    """Context manager for backward passes that accumulate into ``.grad`` (``torch.autograd.backward``
+    / ``Tensor.backward``, the way the reference's executor runs a backward task,
+    src/executors.py:257-296): inside it the fused expert region adds the gradients of leaf
+    parameters whose ``.grad`` already exists to that buffer in the epilogue of the weight-gradient
+    kernels and hands autograd no gradient for them, instead of writing fresh tensors that
+    AccumulateGrad then adds in a separate pass over 3 x E x I x H elements.  Gradient accumulation
+    over microbatches as in src/executors.py:333-343.  Not for ``torch.autograd.grad``, which must
+    return the gradients and leave ``.grad`` alone."""
+
+    def __enter__(self):
+        global _ACCUMULATE_INTO_GRAD
+        self._prev = _ACCUMULATE_INTO_GRAD
+        _ACCUMULATE_INTO_GRAD = True
+        return self
+
+    def __exit__(self, *exc) -> None:
+        global _ACCUMULATE_INTO_GRAD
+        _ACCUMULATE_INTO_GRAD = self._prev
+
+
+def _accumulates_in_place(p) -> bool:
+    """A leaf whose existing .grad the kernels can add to directly."""
+    if p is None or not (p.is_leaf and p.requires_grad):
+        return False
+    g = p.grad
+    return g is not None and g.dtype == p.dtype and g.shape == p.shape and g.is_contiguous() and g.device == p.device
+
+
+def _router_weight_grads(p_gate, p_bias, d_logits, x, w_gate) -> None:
+    """d_w_gate (and d_gate_bias) added to / stored as the parameters' .grad."""
+    # the gate weight and the bias may be at different points of their accumulation
+    # (one of them cleared, the other not); the kernel has one flag for both
+    have_w = p_gate.grad is not None
+    have_b = p_bias is not None and p_bias.grad is not None
+    if p_bias is None or have_w == have_b:
+        gw = p_gate.grad if have_w else torch.empty_like(p_gate)
+        gb = None
+        if p_bias is not None:
+            gb = p_bias.grad if have_b else torch.empty_like(p_bias, dtype=torch.float32)
+        ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=False, d_w_gate=gw, d_gate_bias=gb, accumulate=have_w)
+        p_gate.grad = gw
+        if p_bias is not None:
+            p_bias.grad = gb
+        return
+    gw = torch.empty_like(p_gate)
+    gb = torch.empty_like(p_bias, dtype=torch.float32)
+    ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=False, d_w_gate=gw, d_gate_bias=gb, accumulate=False)
+    p_gate.grad = p_gate.grad.add_(gw) if have_w else gw
+    p_bias.grad = p_bias.grad.add_(gb) if have_b else gb
+
+
 def _can_defer(*params) -> bool:
     return _WGRAD_QUEUE is not None and all(p is None or (p.is_leaf and p.requires_grad) for p in params)
 
@@ -373,30 +439,20 @@ class _ExpertRegionFn(torch.autograd.Function):
             d_x = ops.permute_bwd(d_xs, inv_perm, top_k, addend_f32=d_x32) if need[0] else None
 
             def run_router():
-                # the gate weight and the bias may be at different points of their accumulation
-                # (one of them cleared, the other not); the kernel has one flag for both
-                have_w = p_gate.grad is not None
-                have_b = p_bias is not None and p_bias.grad is not None
-                if p_bias is None or have_w == have_b:
-                    gw = p_gate.grad if have_w else torch.empty_like(p_gate)
-                    gb = None
-                    if p_bias is not None:
-                        gb = p_bias.grad if have_b else torch.empty_like(p_bias, dtype=torch.float32)
-                    ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=False, d_w_gate=gw, d_gate_bias=gb, accumulate=have_w)
-                    p_gate.grad = gw
-                    if p_bias is not None:
-                        p_bias.grad = gb
-                    return
-                gw = torch.empty_like(p_gate)
-                gb = torch.empty_like(p_bias, dtype=torch.float32)
-                ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=False, d_w_gate=gw, d_gate_bias=gb, accumulate=False)
-                p_gate.grad = p_gate.grad.add_(gw) if have_w else gw
-                p_bias.grad = p_bias.grad.add_(gb) if have_b else gb
+                _router_weight_grads(p_gate, p_bias, d_logits, x, w_gate)
 
             _WGRAD_QUEUE.push(run_router)
             return d_x, None, None, None, None, None, None, None, None, (d_out if need[9] else None)
-        side = _side_stream(x.device) if (need[3] or need[4] or need[5]) and _OVERLAP_WGRAD else None
-        if need[3] or need[4] or need[5]:
+        # backward into .grad with gradients already there (a later microbatch of an iteration): the
+        # weight-gradient kernels add to them in their epilogues and autograd gets nothing to add
+        experts_in_place = _ACCUMULATE_INTO_GRAD and all(need[3:6]) and all(_accumulates_in_place(p) for p in ctx.params[2:])
+        p_gate, p_bias = ctx.params[0], ctx.params[1]
+        gate_in_place = (_ACCUMULATE_INTO_GRAD and need[1] and _accumulates_in_place(p_gate)
+                         and (p_bias is None or (need[2] and p_bias.is_leaf and p_bias.requires_grad)))
+        side = _side_stream(x.device) if (need[3] or need[4] or need[5]) and _OVERLAP_WGRAD and not experts_in_place else None
+        if experts_in_place:
+            wgrad(d_w1=ctx.params[2].grad, d_w2=ctx.params[3].grad, d_w3=ctx.params[4].grad, accumulate=True)
+        elif need[3] or need[4] or need[5]:
             if side is not None:
                 side.wait_stream(cur)
                 with torch.cuda.stream(side):
@@ -405,9 +461,14 @@ class _ExpertRegionFn(torch.autograd.Function):
                 d_w1, d_w2, d_w3 = wgrad()
         d_xs = ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
         d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
-        d_wg = torch.empty_like(w_gate) if need[1] else None
-        d_b = torch.empty(E, dtype=torch.float32, device=x.device) if (has_bias and need[2]) else None
-        d_x32 = ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=need[0], d_w_gate=d_wg, d_gate_bias=d_b)
+        if gate_in_place:
+            d_wg = d_b = None
+            d_x32 = ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=need[0], d_w_gate=None, d_gate_bias=None)
+            _router_weight_grads(p_gate, p_bias, d_logits, x, w_gate)
+        else:
+            d_wg = torch.empty_like(w_gate) if need[1] else None
+            d_b = torch.empty(E, dtype=torch.float32, device=x.device) if (has_bias and need[2]) else None
+            d_x32 = ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=need[0], d_w_gate=d_wg, d_gate_bias=d_b)
         d_x = ops.permute_bwd(d_xs, inv_perm, top_k, addend_f32=d_x32) if need[0] else None
         if side is not None:
             cur.wait_stream(side)

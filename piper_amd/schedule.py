@@ -9,9 +9,11 @@ A Piper schedule is a JSON list of directives (src/schedule.py:6-99, src/directi
 The reference lowers them onto a multi-device training DAG.  This module keeps the file format and
 its validation and reduces the meaning to what one GPU can act on: `place` tells how many pipeline
 stages there are, `split` how many microbatches, `order` the sequence of forward / backward passes;
-device lists, streams, `replicate` and `shard` describe other GPUs and are checked for shape
-only.  `device_tasks` turns the result into the `Task` list that `StageExecutor.run` takes, with
-every stage of the file running on the one device.
+device lists, streams and `shard` describe other GPUs and are checked for shape only; of
+`replicate` the one field that also matters on a single device is `bucket_size` (MB,
+src/directives.py:155-169,1620-1621): it cuts the matched stage into parameter buckets
+(`stage_bucket_bytes`, `plan_stage_buckets`).  `device_tasks` turns the result into the `Task`
+list that `StageExecutor.run` takes, with every stage of the file running on the one device.
 
 PASS values (src/directives.py:23-33): "F" forward, "B" fused backward, "BI" backward-input,
 "BW" backward-weight.  A (stage, microbatch) whose backward an order row names as BI / BW runs
@@ -43,6 +45,13 @@ def _check_directive(pos: int, d: Any) -> None:
             raise ValueError(f"{op} directive[{pos}] needs an object field 'filter': {d}")
         if "filters" in d:
             raise ValueError(f"{op} directive[{pos}] takes 'filter', not 'filters': {d}")
+        if op == "replicate" and d.get("bucket_size") is not None:
+            try:
+                mb = int(d["bucket_size"])
+            except (TypeError, ValueError):
+                raise ValueError(f"replicate directive[{pos}]: bucket_size must be a number of MB: {d}") from None
+            if mb <= 0:
+                raise ValueError(f"bucket_size must be > 0 MB, got {mb}")       # src/directives.py:565-566
         if op == "split" and d.get("num_microbatches") == "__MBS__":
             raise ValueError("split.num_microbatches must be a number in the schedule file; the '__MBS__' "
                              "placeholder is not supported")
@@ -118,6 +127,59 @@ def derive_schedule_info(directives: Sequence[dict], schedule_path: str = "") ->
 
 def load_schedule_info(path: str) -> dict[str, Any]:
     return derive_schedule_info(load_schedule_directives(path), path)
+
+
+# ------------------------------------------------------------------------------- bucket sizes
+def _filter_matches_stage(flt: dict, stage: int) -> bool:
+    """The tag match of src/directives.py:46-56 against the tag {PP: stage} of a whole stage: a
+    filter that names another tag than PP selects part of a stage (an EP segment) and does not
+    match the stage as such."""
+    for key, want in flt.items():
+        if key != "PP":
+            return False
+        if want != ANY and int(want) != stage:
+            return False
+    return True
+
+
+def stage_bucket_bytes(directives: Sequence[dict], num_stages: int | None = None) -> list[int | None]:
+    """Per pipeline stage: the parameter-bucket size in bytes that its `replicate` directive asks
+    for (`bucket_size` MB x 1024 x 1024, src/directives.py:567), or None when no replicate
+    directive with a bucket_size matches the stage (the stage then stays one bucket).  The last
+    matching directive wins, as directives are applied in file order (src/directives.py:1607-1621)."""
+    directives = validate_schedule_directives(list(directives))
+    if num_stages is None:      # the stages that the place directives name
+        placed = [int(d["filter"]["PP"]) for d in directives
+                  if d.get("op") == "place" and d["filter"].get("PP", ANY) != ANY]
+        num_stages = 1 + max(placed, default=0)
+    out: list[int | None] = [None] * num_stages
+    for d in directives:
+        if d.get("op") != "replicate" or d.get("bucket_size") is None:
+            continue
+        for stage in range(num_stages):
+            if _filter_matches_stage(d["filter"], stage):
+                out[stage] = int(d["bucket_size"]) * 1024 * 1024
+    return out
+
+
+def plan_stage_buckets(directives: Sequence[dict], stage_node_param_bytes: Sequence[Sequence[Sequence[int]]]):
+    """The compute buckets of every stage of a schedule.
+
+    stage_node_param_bytes[p][i] lists the parameter sizes in bytes of compute node i of stage p (in
+    placeholder order).  Returns (groups, stage_ubids): groups[p] holds the node indices of each
+    bucket of stage p in execution order -- one bucket for a stage without `bucket_size`, the
+    assignment of `planner.bucket_layers` otherwise -- and stage_ubids[p] the running bucket ids,
+    ready for `device_tasks(..., stage_ubids=...)`."""
+    from .planner import bucket_layers
+
+    sizes = stage_bucket_bytes(directives, len(stage_node_param_bytes))
+    groups, stage_ubids, next_id = [], [], 0
+    for nodes, limit in zip(stage_node_param_bytes, sizes):
+        g = [list(range(len(nodes)))] if limit is None else bucket_layers(nodes, limit)
+        groups.append(g)
+        stage_ubids.append(list(range(next_id, next_id + len(g))))
+        next_id += len(g)
+    return groups, stage_ubids
 
 
 # ------------------------------------------------------------------------------- order rows

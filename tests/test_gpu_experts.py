@@ -4,7 +4,7 @@ same bf16 inputs (tolerance 2e-2 of the output's maximum), fp32 results to 1e-5.
 import pytest
 import torch
 
-from conftest import BF16_TOL, F32_TOL, rel_err
+from conftest import BF16_TOL, F32_TOL, rel_err, rel_err_by_expert
 from oracle import moe as O
 from piper_amd import functional as F_
 from piper_amd import ops
@@ -65,6 +65,11 @@ def test_grouped_swiglu_fwd_dgrad_wgrad(dev, dtype, counts, H, I):
     assert rel_err(dx, dx_ref) <= tol
     dw1, dw2, dw3 = ops.grouped_swiglu_wgrad(DY, h, dg, du, X, starts, E)
     assert rel_err(dw1, dw1_ref) <= tol and rel_err(dw2, dw2_ref) <= tol and rel_err(dw3, dw3_ref) <= tol
+    # every expert on its own scale: its rows of y and d_x, its weight gradients
+    for name, got, ref, by_rows in (("y", y, y_ref, True), ("d_x", dx, dx_ref, True), ("d_w1", dw1, dw1_ref, False),
+                                    ("d_w2", dw2, dw2_ref, False), ("d_w3", dw3, dw3_ref, False)):
+        worst, e = rel_err_by_expert(got, ref, counts, rows=by_rows)
+        assert worst <= tol, (name, "expert", e, counts[e], worst)
     for e, c in enumerate(counts):
         if c == 0:  # an expert without rows gets exact zeros, not garbage
             assert float(dw1[e].abs().max()) == 0.0 and float(dw2[e].abs().max()) == 0.0 and float(dw3[e].abs().max()) == 0.0
@@ -111,6 +116,10 @@ def test_scaled_backward_matches_combine_bwd_then_dgrad(dev, dtype, counts, H, I
     assert rel_err(d_xs, dx_ref) <= tol
     dw1, dw2, dw3 = ops.grouped_swiglu_wgrad(DO, hs, d_g, d_u, XT, starts, E, row_map=PERM, row_map_div=K, scaled=True)
     assert rel_err(dw1, dw1_ref) <= tol and rel_err(dw2, dw2_ref) <= tol and rel_err(dw3, dw3_ref) <= tol
+    for name, got, ref, by_rows in (("d_x", d_xs, dx_ref, True), ("d_w1", dw1, dw1_ref, False),
+                                    ("d_w2", dw2, dw2_ref, False), ("d_w3", dw3, dw3_ref, False)):
+        worst, e = rel_err_by_expert(got, ref, counts, rows=by_rows)
+        assert worst <= tol, (name, "expert", e, counts[e], worst)
 
     # the unfused chain on the same inputs
     d_y, d_s2 = ops.combine_bwd(DO, y, PERM, SC)
@@ -242,8 +251,12 @@ def test_transposed_backward_pair_matches_the_plain_pair(dev, counts, H, I):
     y_ref = O.grouped_swiglu(w1r, w2r, w3r, xr, cnt)
     out_ref = torch.zeros(T, H).index_add(0, tok, y_ref * scores.reshape(-1)[perm.long()].unsqueeze(1))
     dw_ref = torch.autograd.grad(out_ref, (w1r, w2r, w3r), d_out.float())
-    for a, b in zip(got, (dw_ref[0], dw_ref[1], dw_ref[2])):
+    for a, b, name in zip(got, (dw_ref[0], dw_ref[1], dw_ref[2]), ("d_w1", "d_w2", "d_w3")):
         assert rel_err(a, b) <= BF16_TOL
+        # every expert on its own scale: a one-row expert's gradient is a few per cent of the
+        # largest one and would hide behind the whole-tensor maximum
+        worst, e = rel_err_by_expert(a, b, counts, rows=False)
+        assert worst <= BF16_TOL, (name, "expert", e, counts[e], worst)
     # accumulate: adds to what is there, twice gives 2x (+ one rounding)
     acc = [t.clone() for t in got]
     ops.grouped_swiglu_wgrad_scaled_t(DO, hsT, d_gT, d_uT, XT, starts, E, row_map=PERM, row_map_div=K,

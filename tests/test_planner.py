@@ -144,3 +144,67 @@ def test_lifetimes_adjacent_backwards_share_one_reduction():
     # explicit edges override the serial default: no link between the two backward tasks
     lt = plan_zero_lifetimes(tasks, direct_deps={(0, 1), (1, 2), (0, 3)})
     assert lt[2].reduce_grads_after and lt[3].reduce_grads_after
+
+
+def test_assignment_equals_the_restated_reference_rule_on_random_inputs():
+    """plan_param_buckets against oracle.planner.assign_buckets (a line-by-line restatement of
+    src/bucket.py:76-128) on 20,000 random (sizes, use ranges, threshold): the same buckets with the
+    same spans in the same execution order.  Inside a bucket that the merge stage joined, the
+    member order may differ (the reference uses it for a log line only, src/bucket.py:133-141), so
+    members are compared as sets."""
+    from oracle.planner import assign_buckets
+
+    rng = random.Random(1234)
+    reordered = 0
+    for case in range(20000):
+        n = rng.randint(1, 14)
+        sizes = [rng.choice((0, 1, 3, 7, 10, 25, 40)) if rng.random() < 0.7 else rng.randint(0, 60) for _ in range(n)]
+        limit = rng.randint(1, 80)
+        nodes = rng.randint(1, 12)
+        ranges = []
+        for _ in range(n):
+            a = rng.randrange(nodes)
+            b = a if rng.random() < 0.6 else rng.randrange(a, nodes)
+            ranges.append((a, b))
+        if rng.random() < 0.3:      # the common case: parameters in the order their nodes use them
+            ranges.sort()
+        got = plan_param_buckets(sizes, ranges, limit)
+        want = assign_buckets(sizes, ranges, limit)
+        assert [(b.first_use, b.last_use, sorted(b.members)) for b in got] == [(f, l, sorted(m)) for f, l, m in want], \
+            (case, sizes, ranges, limit)
+        reordered += any(b.members != m for b, (_, _, m) in zip(got, want))
+    assert reordered < 20000 // 4
+
+
+def test_bucket_size_of_a_schedule_cuts_the_stage():
+    """replicate.bucket_size (MB) -> bytes per stage -> node groups -> bucket ids for device_tasks."""
+    from piper_amd.schedule import device_tasks, plan_stage_buckets, stage_bucket_bytes
+
+    mib = 1024 * 1024
+    sched = [
+        {"op": "place", "filter": {"PP": 0}, "devices": [0]},
+        {"op": "place", "filter": {"PP": 1}, "devices": [1]},
+        {"op": "replicate", "filter": {"PP": 0}, "devices": [0, 2], "reduce_stream": "dp_stream", "bucket_size": 2},
+        {"op": "replicate", "filter": {"PP": 1}, "devices": [1, 3]},
+        {"op": "shard", "filter": {"PP": 0, "EP": "*"}, "devices": [0, 2]},
+        {"op": "split", "filter": {}, "dim_name": "MB", "num_microbatches": 2},
+    ]
+    assert stage_bucket_bytes(sched) == [2 * mib, None]
+    # stage 0: four nodes of 1.5 MiB of parameters each -> one node per bucket; stage 1 stays whole
+    node = [mib, mib // 2]
+    groups, ubids = plan_stage_buckets(sched, [[node] * 4, [node] * 3])
+    assert groups == [[[0], [1], [2], [3]], [[0, 1, 2]]]
+    assert ubids == [[0, 1, 2, 3], [4]]
+    tasks = device_tasks(sched, stage_ubids=ubids)
+    fwd0 = [t.ubid for t in tasks if t.type is TaskType.FWD and t.mb == 0]
+    bwd0 = [t.ubid for t in tasks if t.type is TaskType.BWD and t.mb == 0]
+    assert fwd0 == [0, 1, 2, 3, 4] and bwd0 == [4, 3, 2, 1, 0]
+    # a wildcard stage filter reaches every stage, a later directive overrides an earlier one
+    both = sched + [{"op": "replicate", "filter": {"PP": "*"}, "devices": [0, 1], "bucket_size": 100}]
+    assert stage_bucket_bytes(both) == [100 * mib, 100 * mib]
+    # a filter on part of a stage (an EP segment) does not set the stage's bucket size
+    ep = [sched[0], {"op": "replicate", "filter": {"PP": 0, "EP": 0}, "devices": [0], "bucket_size": 7}]
+    assert stage_bucket_bytes(ep) == [None]
+    for bad in (0, -3, "x"):
+        with pytest.raises(ValueError):
+            stage_bucket_bytes([sched[0], {"op": "replicate", "filter": {"PP": 0}, "devices": [0], "bucket_size": bad}])

@@ -89,3 +89,55 @@ def test_static_sort_rejects_inputs_beyond_its_scratch(dev):
     torch.cuda.synchronize()
     assert o["counts"][0].item() == A_ok and o["starts"][E].item() == A_ok
     assert torch.equal(o["perm"], torch.arange(A_ok, dtype=torch.int32, device=dev))
+
+
+def test_static_sort_recorded_into_a_hip_graph(dev):
+    """Two static sorts recorded into one HIP graph (after pk_init on the device, as the header
+    asks: a symbol look-up is not legal while a stream is capturing) and replayed with new inputs,
+    with eager work between the replays; every replay against pk_sort_by_expert on the same inputs."""
+    lib = _lib.load()
+    _lib.init_device()
+    g = torch.Generator().manual_seed(3)
+    shapes = [(4096 * 8, 128), (1000 * 2 + 3, 8)]
+    inputs = [torch.zeros(A, dtype=torch.int32, device=dev) for A, _ in shapes]
+    outs = [_outputs(A, E, dev) for A, E in shapes]
+
+    def fill():
+        for buf, (A, E) in zip(inputs, shapes):
+            buf.copy_(torch.randint(0, E, (A,), generator=g, dtype=torch.int32))
+
+    def static_sorts():
+        stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        for buf, o, (A, E) in zip(inputs, outs, shapes):
+            rc = lib.pk_sort_by_expert_static(_p(buf), A, E, _p(o["counts"]), _p(o["starts"]), _p(o["perm"]),
+                                              _p(o["inv_perm"]), _p(o["order"]), stream)
+            assert rc == 0
+
+    fill()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        static_sorts()                     # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    print("[case] static sort under graph capture", flush=True)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_sorts()
+    for rep in range(3):
+        fill()
+        for o in outs:
+            for t in o.values():
+                t.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        for buf, o, (A, E) in zip(inputs, outs, shapes):       # eager, between the replays
+            ref = _outputs(A, E, dev)
+            ws = torch.empty(max(int(lib.pk_sort_workspace_bytes(A, E)), 4), dtype=torch.uint8, device=dev)
+            rc = lib.pk_sort_by_expert(_p(buf), A, E, _p(ref["counts"]), _p(ref["starts"]), _p(ref["perm"]),
+                                       _p(ref["inv_perm"]), _p(ref["order"]), _p(ws), ws.numel(),
+                                       C.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+            assert rc == 0
+            torch.cuda.synchronize()
+            for name in ref:
+                assert torch.equal(ref[name], o[name]), f"replay {rep}: {name} (A={A}, E={E})"
