@@ -249,21 +249,25 @@ def _host_threads() -> int:
 
 
 def cpu_baseline(cfg):
-    """The CPU oracle (un-padded per-expert loop, fp32) on a bounded sample of the same workload:
-    the first tokens of the microbatch with the full set of experts.  The fp32 copies of the
-    inputs are made once, outside the timed passes."""
+    """The CPU oracle (un-padded per-expert loop, fp32) on a bounded sample of the same workload: one
+    eighth of the experts with one eighth of the tokens, so that an expert receives as many rows as in
+    the full microbatch and every GEMM keeps its shape; the full microbatch is eight such samples
+    (the time of a pass goes into the per-expert matmuls and into writing the weight gradients,
+    both proportional to the number of experts).  The fp32 copies of the inputs are made once,
+    outside the timed passes."""
     import torch
 
     from oracle import moe as O
     from piper_amd.configs import make_expert_region_inputs
 
     cores = _host_threads()
-    sample_tokens = min(cfg.tokens, 512)
+    frac = 8 if cfg.num_experts % 8 == 0 and cfg.num_experts // 8 >= cfg.top_k and cfg.tokens % 8 == 0 else 1
+    n_tok, n_exp = cfg.tokens // frac, cfg.num_experts // frac
     inp = make_expert_region_inputs(cfg)
     names = ("x", "w_gate", "w1", "w2", "w3")
-    leaves = {k: (inp[k][:sample_tokens] if k == "x" else inp[k]).float().requires_grad_(True) for k in names}
-    d_out = inp["d_out"][:sample_tokens].float()
-    bias = inp["gate_bias"]
+    leaves = {k: (inp[k][:n_tok] if k == "x" else inp[k][:n_exp]).float().requires_grad_(True) for k in names}
+    d_out = inp["d_out"][:n_tok].float()
+    bias = inp["gate_bias"][:n_exp] if inp["gate_bias"] is not None else None
 
     def one():
         out, _ = O.moe_forward(leaves["x"], leaves["w_gate"], bias, leaves["w1"], leaves["w2"], leaves["w3"], cfg.top_k,
@@ -271,8 +275,9 @@ def cpu_baseline(cfg):
         torch.autograd.grad(out, list(leaves.values()), d_out)
 
     t = _median_of_3(one)
-    return {"value": sample_tokens / t, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"first {sample_tokens} of {cfg.tokens} tokens, all {cfg.num_experts} experts, fp32 per-expert loop, "
+    return {"value": n_tok / t, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"first {n_tok} of {cfg.tokens} tokens routed over the first {n_exp} of {cfg.num_experts} experts "
+                      f"({n_tok * cfg.top_k // n_exp} rows per expert on average, as in the full microbatch), fp32 per-expert loop, "
                       f"fwd+bwd, median of 3 after 1 warm-up ({t:.2f} s per pass)"}
 
 

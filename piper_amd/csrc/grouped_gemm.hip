@@ -557,6 +557,34 @@ struct Stage32 {
     }
     return nrows >= 32 ? NP : nrows <= 0 ? 0 : (nrows + RPP - 1) / RPP;
   }
+  // All 32 rows of the staged tile added to values fetched earlier (old[q]: what flush would read
+  // at dst for pass q -- rows q * RPP + lane / CH, 16-byte piece lane % CH) and stored: fp32 add, one
+  // rounding of the sum.  Returns the number of store instructions issued.
+  template <bool STREAM>
+  __device__ static __forceinline__ int flush_add(const char* buf, bf16_t* dst, int64_t ldc, const u32x4_t (&old)[32 / (64 / CH)],
+                                                  int lane = threadIdx.x & 63) {
+    constexpr int RPP = 64 / CH, NP = 32 / RPP;
+    const int lr = lane / CH, lc = lane % CH;
+    u32x4_t v[NP];
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      const int r = q * RPP + lr;
+      v[q] = *reinterpret_cast<const u32x4_t*>(buf + r * ROWB + (((lc ^ r) & (CH - 1)) << 4));
+    }
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      const int r = q * RPP + lr;
+      const bf16x8_t a = __builtin_bit_cast(bf16x8_t, v[q]);
+      const bf16x8_t o = __builtin_bit_cast(bf16x8_t, old[q]);
+      bf16x8_t sum;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) sum[t] = (bf16_t)((float)a[t] + (float)o[t]);
+      u32x4_t* g = reinterpret_cast<u32x4_t*>(dst + (int64_t)r * ldc + lc * 8);
+      if (STREAM) __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, sum), g);
+      else *g = __builtin_bit_cast(u32x4_t, sum);
+    }
+    return NP;
+  }
   // The staged tile transposed: element (r, c) goes to dstT[c * ldt + r] (ldt = 32 for the blocked
   // transposed copies), rows in groups of 8 (16 bytes per lane).  With nrows > 0 all 32 rows are
   // written: the caller stages zeros in rows nrows..31, and the consumer finds zeros up to the end
@@ -1528,7 +1556,7 @@ struct WgradKcParams {
 //  * A workgroup requests the first k-tiles of its next unit before the epilogue of the current one
 //    (or, when the next unit is known in time, as the last requests of the k-loop), and its
 //    stores do not hold up the next unit's loads.
-template <int WMW, int WNW, bool A_KC, bool DYNAMIC>
+template <int WMW, int WNW, bool A_KC, bool DYNAMIC, bool ACCUMULATE>
 __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_pp_kernel(const WgradKcParams p) {
   constexpr int BM = 256, BN = 256, BK = 32, NS = 4;
   constexpr bool B_KC = !A_KC;
@@ -1866,18 +1894,39 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_pp_kernel(const WgradKcP
         issue_prologue(cur);
       }
     };
-    // an accumulating epilogue reads the old gradients, and a wave waits for a load only together
-    // with everything it requested before it: there the requests go behind the epilogue
-    if (!p.accumulate || chained) prefetch_next();
-
-    if (!(p.accumulate && nkt == 0)) {
-      const WgradKcProblem& q = p.prob[cur_u.q];
-      bf16_t* const C = q.C + (int64_t)cur_u.e * p.M * p.N + (int64_t)(cur_u.mt * BM + wm * WTM) * p.N + cur_u.nt * BN + wn * WTN;
+    // An accumulating epilogue (ACCUMULATE, a kernel of its own: the registers below would
+    // otherwise be spilled around the k-loop of the plain one) adds to the gradients that are there.
+    // Behind the requests for the next unit's first k-tiles a wave requests the old values of
+    // OLD_BATCH of its 32 x 64 chunks at a time (the fragment registers are dead here) and only then
+    // stages and stores them: the old values come back under one memory round trip per batch
+    // instead of one per chunk.  They are younger than the next unit's first tiles, like the stores.
+    constexpr int NCH = TM * (TN / 2), OLD_NP = 4, OLD_BATCH = 2;
+    static_assert(St::CH == 8 && NCH % OLD_BATCH == 0, "a staged chunk is 32 rows of eight 16-byte pieces");
+    const WgradKcProblem& q = p.prob[cur_u.q];
+    bf16_t* const C = q.C + (int64_t)cur_u.e * p.M * p.N + (int64_t)(cur_u.mt * BM + wm * WTM) * p.N + cur_u.nt * BN + wn * WTN;
+    const bool write_tile = !(ACCUMULATE && nkt == 0);      // nothing to add for an expert without rows
+    prefetch_next();
+    if (write_tile) {
       const int lrow = lane & 31, lq = 4 * (lane >> 5);
+      const int lr = lane / St::CH, lc = lane % St::CH;
+      auto chunk_dst = [&](int c) { return C + (int64_t)(32 * (c / (TN / 2))) * p.N + 64 * (c % (TN / 2)); };
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+      for (int c0 = 0; c0 < NCH; c0 += OLD_BATCH) {
+        u32x4_t old[ACCUMULATE ? OLD_BATCH : 1][OLD_NP];
+        if constexpr (ACCUMULATE) {
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int jh = 0; jh < TN; jh += 2) {
+          for (int c = 0; c < OLD_BATCH; ++c)
+#pragma unroll
+            for (int qq = 0; qq < OLD_NP; ++qq)
+              old[c][qq] = __builtin_nontemporal_load(
+                  reinterpret_cast<const u32x4_t*>(chunk_dst(c0 + c) + (int64_t)(qq * 8 + lr) * p.N + lc * 8));
+          st_after += OLD_BATCH * OLD_NP;
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int c = c0; c < c0 + OLD_BATCH; ++c) {
+          const int i = c / (TN / 2), jh = 2 * (c % (TN / 2));
 #pragma unroll
           for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
@@ -1885,13 +1934,12 @@ __global__ __launch_bounds__(64 * WMW * WNW) void wgrad_pp_kernel(const WgradKcP
               St::put(sbuf, lrow, 32 * jj + 8 * qd + lq,
                       pack4(acc[i][jh + jj][4 * qd], acc[i][jh + jj][4 * qd + 1], acc[i][jh + jj][4 * qd + 2], acc[i][jh + jj][4 * qd + 3]));
           wave_lds_fence();
-          bf16_t* const dst = C + (int64_t)(32 * i) * p.N + 32 * jh;
-          if (p.accumulate) St::template flush<true, true>(sbuf, dst, p.N, 32);
-          else st_after += St::template flush<false, true>(sbuf, dst, p.N, 32);
+          if constexpr (ACCUMULATE) st_after += St::template flush_add<true>(sbuf, chunk_dst(c), p.N, old[c - c0]);
+          else st_after += St::template flush<false, true>(sbuf, chunk_dst(c), p.N, 32);
           wave_lds_fence();
         }
+      }
     }
-    if (p.accumulate && !chained) prefetch_next();
     if (!has_next) break;
     cur_u = nxt_u;
     par ^= 1;
@@ -2538,10 +2586,16 @@ int pk_grouped_swiglu_wgrad_scaled_t(const void* d_out, const void* hsT, const v
       if (!p.sched) return PK_ERR_UNSUPPORTED;
     }
     const int id = a_kc ? pk_timing::K_SWIGLU_WGRAD_W13 : pk_timing::K_SWIGLU_WGRAD_W2;
-    if (a_kc && dynamic) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_pp_kernel<2, 4, true, true>), grid, block, 0, s, p);
-    else if (a_kc) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_pp_kernel<2, 4, true, false>), grid, block, 0, s, p);
-    else if (dynamic) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_pp_kernel<4, 2, false, true>), grid, block, 0, s, p);
-    else PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_pp_kernel<4, 2, false, false>), grid, block, 0, s, p);
+#define PK_WGRAD_PP(WMW, WNW, AKC, DYN)                                                                         \
+  do {                                                                                                          \
+    if (p.accumulate) PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_pp_kernel<WMW, WNW, AKC, DYN, true>), grid, block, 0, s, p);   \
+    else PK_LAUNCH_NOCHECK(id, s, (mf::wgrad_pp_kernel<WMW, WNW, AKC, DYN, false>), grid, block, 0, s, p);               \
+  } while (0)
+    if (a_kc && dynamic) PK_WGRAD_PP(2, 4, true, true);
+    else if (a_kc) PK_WGRAD_PP(2, 4, true, false);
+    else if (dynamic) PK_WGRAD_PP(4, 2, false, true);
+    else PK_WGRAD_PP(4, 2, false, false);
+#undef PK_WGRAD_PP
     PK_RETURN_IF_LAUNCH_FAILED();
     return PK_OK;
   };
