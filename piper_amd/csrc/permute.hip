@@ -22,6 +22,20 @@ struct RowIO {
       f[0] = pk_to_float<T>(row[v]);
     }
   }
+  // the same load for rows that are read once and are too many to stay in a cache: a streaming
+  // (nontemporal) load keeps them from pushing out what other kernels left there (measured on
+  // 537 MB of gathered rows: 5.0 -> 5.5 TB/s; on 134 MB, which the memory-side cache holds, the
+  // ordinary load is the faster one, 6.5 against 6.0 TB/s)
+  __device__ static __forceinline__ void load_once(const T* row, int64_t v, float (&f)[PkVec16<T>::N]) {
+    if (VEC) {
+      PkVec16<T> x;
+      x.v = __builtin_nontemporal_load(reinterpret_cast<const decltype(x.v)*>(row + v * N));
+#pragma unroll
+      for (int i = 0; i < N; ++i) f[i] = x.get(i);
+    } else {
+      f[0] = pk_to_float<T>(row[v]);
+    }
+  }
   __device__ static __forceinline__ void store(T* row, int64_t v, const float (&f)[PkVec16<T>::N]) {
     if (VEC) {
       PkVec16<T> x;
@@ -59,7 +73,7 @@ __global__ __launch_bounds__(kRowThreads) void permute_fwd_kernel(
 // memory behind the load of its index.  Indices and weights of up to KB terms are fetched first
 // (wave-uniform addresses), then the KB row loads are issued together and summed in k order (the
 // same sum, term by term, as one load at a time).
-template <typename T, bool VEC>
+template <typename T, bool VEC, bool STREAM>
 __global__ __launch_bounds__(kRowThreads) void gather_reduce_kernel(
     const T* __restrict__ rows, const int32_t* __restrict__ inv_perm,
     const float* __restrict__ weights, const float* __restrict__ addend, const T* __restrict__ residual,
@@ -84,7 +98,10 @@ __global__ __launch_bounds__(kRowThreads) void gather_reduce_kernel(
       }
       float f[KB][N];
 #pragma unroll
-      for (int j = 0; j < KB; ++j) IO::load(rows + p[j] * H, v, f[j]);
+      for (int j = 0; j < KB; ++j) {
+        if (STREAM) IO::load_once(rows + p[j] * H, v, f[j]);
+        else IO::load(rows + p[j] * H, v, f[j]);
+      }
 #pragma unroll
       for (int j = 0; j < KB; ++j) {
         if (k0 + j < K) {
@@ -379,13 +396,21 @@ static int gather_reduce(const void* rows, int dtype, const int32_t* inv_perm, c
   const bool vec = vec_ok(dtype, H, {rows, out, residual});
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)T);
+  // rows that do not fit the memory-side cache (256 MB) are streamed
+  const bool stream_rows = T * K * H * (int64_t)pk_dtype_size(dtype) > (int64_t)192 * 1024 * 1024;
+#define PK_GATHER_REDUCE(TYPE, VECF, STREAMF)                                                                          \
+  PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<TYPE, VECF, STREAMF>), grid, dim3(kRowThreads), 0, s, \
+                    (const TYPE*)rows, inv_perm, weights, addend, (const TYPE*)residual, (TYPE*)out, H, (int)K)
   if (dtype == PK_BF16) {
-    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<bf16_t, true>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)rows, inv_perm, weights, addend, (const bf16_t*)residual, (bf16_t*)out, H, (int)K);
-    else PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<bf16_t, false>), grid, dim3(kRowThreads), 0, s, (const bf16_t*)rows, inv_perm, weights, addend, (const bf16_t*)residual, (bf16_t*)out, H, (int)K);
+    if (vec && stream_rows) PK_GATHER_REDUCE(bf16_t, true, true);
+    else if (vec) PK_GATHER_REDUCE(bf16_t, true, false);
+    else PK_GATHER_REDUCE(bf16_t, false, false);
   } else {
-    if (vec) PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<float, true>), grid, dim3(kRowThreads), 0, s, (const float*)rows, inv_perm, weights, addend, (const float*)residual, (float*)out, H, (int)K);
-    else PK_LAUNCH_NOCHECK(pk_timing::K_GATHER_REDUCE, s, (gather_reduce_kernel<float, false>), grid, dim3(kRowThreads), 0, s, (const float*)rows, inv_perm, weights, addend, (const float*)residual, (float*)out, H, (int)K);
+    if (vec && stream_rows) PK_GATHER_REDUCE(float, true, true);
+    else if (vec) PK_GATHER_REDUCE(float, true, false);
+    else PK_GATHER_REDUCE(float, false, false);
   }
+#undef PK_GATHER_REDUCE
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
 }
