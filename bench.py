@@ -203,6 +203,22 @@ def bench_bucket(steps: int, warmup: int):
     torch.cuda.synchronize()
     records = _lib.timing_collect()
     _lib.timing_enable(False)
+    # the same step with the pack folded into the optimizer kernel (the last microbatch of an
+    # iteration, or the only one): bf16 gradients read straight from the tensors, no fp32 gradient bucket
+    def fused_step():
+        state["step"] += 1
+        ops.adamw_fused_packed(master, m, v, None, grads, offs, numels, step=state["step"], lr=ADAMW["lr"],
+                               beta1=ADAMW["betas"][0], beta2=ADAMW["betas"][1], eps=ADAMW["eps"],
+                               weight_decay=ADAMW["weight_decay"], shadow=shadow)
+
+    for _ in range(warmup):
+        fused_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fused_step()
+    torch.cuda.synchronize()
+    fused_elapsed = time.perf_counter() - t0
     n_elems = sum(numels)
     pack_ms = [ms for k, ms in records if k == "bucket_pack"]
     adam_ms = [ms for k, ms in records if k == "adamw"]
@@ -225,6 +241,12 @@ def bench_bucket(steps: int, warmup: int):
                      "frac": agg_gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
                      "bytes_per_step": pack_bytes + adam_bytes},
+        # one launch instead of two: its own algorithmic bytes (read bf16 grad 2 + p,m,v 12; write p,m,v 12 +
+        # bf16 parameter 2 = 28 per element), and the time it takes against the two-kernel step
+        "fused_last_pack": {"ms_per_step": fused_elapsed / steps * 1e3, "bytes_per_element": 28,
+                            "GB/s": 28.0 * n_elems * steps / fused_elapsed / 1e9,
+                            "frac": 28.0 * n_elems * steps / fused_elapsed / 1e9 / HBM_PEAK_GBS,
+                            "vs_two_kernels": (fused_elapsed / steps) / (elapsed / steps)},
     }
 
 

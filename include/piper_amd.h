@@ -364,6 +364,26 @@ PK_API int pk_adamw_fused(float* master, float* exp_avg, float* exp_avg_sq, floa
                    float weight_decay, int64_t step, float grad_scale, int zero_grad,
                    pk_stream_t stream);
 
+/* pk_bucket_pack of the LAST microbatch's gradients folded into pk_adamw_fused: the gradient of
+ * bucket element offsets[i] + j is flat_grad[offsets[i] + j] (fp32, what earlier microbatches packed;
+ * flat_grad may be NULL = zero) plus grads[i][j] (grad_dtype; grads[i] may be NULL = the tensor
+ * received no gradient in the last microbatch), added in fp32 exactly as pk_bucket_pack with
+ * accumulate would have stored it, so master, moments and the bf16 parameter bucket come out
+ * bit-identical to pk_bucket_pack(accumulate) followed by pk_adamw_fused, while the fp32 gradient
+ * bucket is neither written nor read again (28 bytes per element with one microbatch, against 6 + 30).
+ * grads / offsets / numels are HOST arrays of n entries as in pk_bucket_pack; every tensor is
+ * stepped, with or without a gradient of its own.  Bucket elements that belong to no tensor
+ * (alignment padding) are left as they are; in a bucket built by pk_bucket_plan they hold zeros in
+ * every buffer and an AdamW step leaves such elements at zero.  zero_grad != 0 clears the flat_grad
+ * elements of the tensors.  shadow (may be NULL) must be bf16.  Replaces the last call of
+ * ParamStorage.accumulate_zero_param_grads_to_flat (src/runtime.py:249-282) together with
+ * step_zero_shard_optimizers (src/runtime.py:454-484). */
+PK_API int pk_adamw_fused_packed(float* master, float* exp_avg, float* exp_avg_sq, float* flat_grad,
+                          const void* const* grads, const int64_t* offsets, const int64_t* numels, int64_t n,
+                          int grad_dtype, void* shadow, int shadow_dtype, float lr, float beta1, float beta2,
+                          float eps, float weight_decay, int64_t step, float grad_scale, int zero_grad,
+                          pk_stream_t stream);
+
 /* ------------------------------------------------------------- kernel timing
  * Measurement aid with no counterpart in the reference: when enabled, every kernel launch of
  * the library is bracketed by two hipEventRecord calls on its stream.  pk_timing_collect

@@ -72,6 +72,8 @@ SIGNATURES = {
     "pk_bucket_zero": (_c_int, [_p, _c_i64, _p]),
     "pk_adamw_fused": (_c_int, [_p, _p, _p, _p, _p, _c_int, _c_i64, _c_f32, _c_f32, _c_f32, _c_f32,
                                 _c_f32, _c_i64, _c_f32, _c_int, _p]),
+    "pk_adamw_fused_packed": (_c_int, [_p, _p, _p, _p, _p, _p, _p, _c_i64, _c_int, _p, _c_int, _c_f32, _c_f32, _c_f32,
+                                       _c_f32, _c_f32, _c_i64, _c_f32, _c_int, _p]),
     "pk_timing_enable": (_c_int, [_c_int]),
     "pk_timing_collect": (_c_i64, [_p, _p, _c_i64]),
     "pk_timing_select": (_c_int, [_c_int]),

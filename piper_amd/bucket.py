@@ -52,6 +52,10 @@ class BucketState:
     # no such field: its flatten concatenates the parameters of a bucket whatever their dtype
     # (src/actor.py:534).
     companions: list = field(default_factory=list)
+    # Gradients of the last microbatch that were NOT packed (ParamStorage.hold_param_grads): one
+    # entry per param_view_spec, consumed by the optimizer step, which adds them to the bucket's
+    # gradient inside the AdamW kernel.
+    pending_grads: list | None = None
 
     def with_companions(self) -> list:
         return [self] + list(self.companions)
@@ -271,6 +275,26 @@ class ParamStorage:
             for param, *_ in specs:
                 param.grad = None
 
+    def hold_param_grads(self, ubid, stream: torch.cuda.Stream | None = None) -> None:
+        """In place of the LAST accumulate_zero_param_grads_to_flat of an iteration: keep the
+        per-tensor gradients of the bucket as they are and drop them from the parameters.  The
+        optimizer step then reads them directly (FusedAdamW.step_packed), which saves writing them
+        into the fp32 bucket and reading them back.  With an optimizer that has no step_packed the
+        step packs them first."""
+        if ubid is None or ubid not in self.stages.zero_managed_ubids:
+            return
+        for bucket in self.stages.bucket(ubid).with_companions():
+            held = []
+            for param, *_ in bucket.param_view_specs:
+                g = param.grad
+                if g is not None:
+                    g = g.detach()
+                    if stream is not None:
+                        g.record_stream(stream)
+                held.append(g)
+                param.grad = None
+            bucket.pending_grads = held
+
     def alloc_full_params(self, ubid) -> None:
         """Unflatten (src/runtime.py:312-352): make every parameter a view of the flat bucket."""
         self.wait_pending_free(self.pending_param_frees, ubid)
@@ -323,9 +347,19 @@ class ParamStorage:
             opt = bucket.shard_optimizer
             if opt is None or bucket.reduce_scatter_grads is None:
                 continue
+            held, bucket.pending_grads = bucket.pending_grads, None
             with torch.cuda.stream(stream):
-                bucket.shard_param.grad = bucket.reduce_scatter_grads
-                opt.step()
+                if held is not None and hasattr(opt, "step_packed") and len({g.dtype for g in held if g is not None}) <= 1:
+                    specs = bucket.param_view_specs
+                    opt.step_packed(bucket.shard_param, held, [s[1] for s in specs], [s[2] for s in specs],
+                                    bucket.reduce_scatter_grads)
+                else:
+                    if held is not None:      # an optimizer without the fused entry: pack first
+                        for (param, *_), g in zip(bucket.param_view_specs, held):
+                            param.grad = g
+                        self._pack_one(bucket, stream)
+                    bucket.shard_param.grad = bucket.reduce_scatter_grads
+                    opt.step()
             bucket.shard_param.grad = None
             for param, *_ in bucket.param_view_specs:
                 param.grad = None

@@ -277,6 +277,108 @@ __global__ __launch_bounds__(kStreamThreads) void adamw_kernel(
   }
 }
 
+// AdamW with the last gradient pack folded in: the gradient of an element is what the fp32 bucket
+// holds (earlier microbatches; optional) plus the per-tensor gradient of the last microbatch, read
+// in its own dtype straight from the tensor.  One block updates kAdamPackChunk elements of one
+// tensor (four per lane: one 16-byte vector per fp32 stream, as in adamw_kernel); bucket elements
+// that belong to no tensor (alignment padding) are not touched.
+constexpr int kAdamPackChunk = kStreamThreads * 4;
+
+template <typename TG, typename TSH, bool SHADOW, bool FLAT, bool ZERO>
+__global__ __launch_bounds__(kStreamThreads) void adamw_packed_kernel(
+    const PackArgs args, float* __restrict__ master, float* __restrict__ exp_avg, float* __restrict__ exp_avg_sq,
+    float* __restrict__ flat_grad, TSH* __restrict__ shadow, const AdamArgs a) {
+  int lo = 0, hi = args.n;  // blk_start[lo] <= blockIdx.x < blk_start[hi]
+  const int b = blockIdx.x;
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (args.blk_start[mid] <= b) lo = mid; else hi = mid;
+  }
+  const int ti = lo;
+  const int64_t numel = args.numel[ti];
+  const int64_t base = (int64_t)(b - args.blk_start[ti]) * kAdamPackChunk;
+  const int64_t cnt = (numel - base) < (int64_t)kAdamPackChunk ? (numel - base) : (int64_t)kAdamPackChunk;
+  const TG* src = args.src[ti] ? reinterpret_cast<const TG*>(args.src[ti]) + base : nullptr;
+  const int64_t o = args.off[ti] + base;
+  const bool src_vec = ((uintptr_t)src & (sizeof(TG) * 4 - 1)) == 0;
+  const int64_t e = (int64_t)threadIdx.x * 4;
+  if (e + 4 <= cnt && ((o & 3) == 0)) {
+    floatx4_t p = __builtin_nontemporal_load(reinterpret_cast<floatx4_t*>(master + o + e));
+    floatx4_t m = __builtin_nontemporal_load(reinterpret_cast<floatx4_t*>(exp_avg + o + e));
+    floatx4_t v = __builtin_nontemporal_load(reinterpret_cast<floatx4_t*>(exp_avg_sq + o + e));
+    floatx4_t g = {0.f, 0.f, 0.f, 0.f};
+    if (FLAT) g = __builtin_nontemporal_load(reinterpret_cast<floatx4_t*>(flat_grad + o + e));
+    if (src) {
+      float t[4];
+      if (src_vec) {
+        if (sizeof(TG) == 2) {
+          const bf16x4_t r = __builtin_nontemporal_load(reinterpret_cast<const bf16x4_t*>(src + e));
+#pragma unroll
+          for (int j = 0; j < 4; ++j) t[j] = (float)r[j];
+        } else {
+          const floatx4_t r = __builtin_nontemporal_load(reinterpret_cast<const floatx4_t*>(src + e));
+#pragma unroll
+          for (int j = 0; j < 4; ++j) t[j] = r[j];
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t[j] = pk_to_float<TG>(src[e + j]);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) g[j] = g[j] + t[j];      // bucket + tensor: the sum the pack kernel stores
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float pj = p[j], mj = m[j], vj = v[j];
+      adam_update(pj, mj, vj, g[j], a);
+      p[j] = pj; m[j] = mj; v[j] = vj;
+    }
+    __builtin_nontemporal_store(p, reinterpret_cast<floatx4_t*>(master + o + e));
+    __builtin_nontemporal_store(m, reinterpret_cast<floatx4_t*>(exp_avg + o + e));
+    __builtin_nontemporal_store(v, reinterpret_cast<floatx4_t*>(exp_avg_sq + o + e));
+    if (SHADOW) {
+      if (sizeof(TSH) == 2) {
+        bf16x4_t sh;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sh[j] = (bf16_t)p[j];
+        __builtin_nontemporal_store(sh, reinterpret_cast<bf16x4_t*>(shadow + o + e));
+      } else {
+        __builtin_nontemporal_store(p, reinterpret_cast<floatx4_t*>(shadow + o + e));
+      }
+    }
+    if (FLAT && ZERO) {
+      floatx4_t z = {0.f, 0.f, 0.f, 0.f};
+      __builtin_nontemporal_store(z, reinterpret_cast<floatx4_t*>(flat_grad + o + e));
+    }
+  } else {
+    for (int64_t i = e; i < cnt && i < e + 4; ++i) {     // a tensor's last elements, unaligned offsets
+      float pj = master[o + i], mj = exp_avg[o + i], vj = exp_avg_sq[o + i];
+      float gj = FLAT ? flat_grad[o + i] : 0.f;
+      if (src) gj = gj + pk_to_float<TG>(src[i]);
+      adam_update(pj, mj, vj, gj, a);
+      master[o + i] = pj; exp_avg[o + i] = mj; exp_avg_sq[o + i] = vj;
+      if (SHADOW) shadow[o + i] = pk_from_float<TSH>(pj);
+      if (FLAT && ZERO) flat_grad[o + i] = 0.f;
+    }
+  }
+}
+
+AdamArgs make_adam_args(float lr, float beta1, float beta2, float eps, float weight_decay, int64_t step, float grad_scale) {
+  // scalar prologue in double, as torch does on the host (python floats)
+  const double bc1 = 1.0 - pow((double)beta1, (double)step);
+  const double bc2 = 1.0 - pow((double)beta2, (double)step);
+  AdamArgs a;
+  a.decay = (float)(1.0 - (double)lr * (double)weight_decay);
+  a.one_m_b1 = (float)(1.0 - (double)beta1);
+  a.beta2 = beta2;
+  a.one_m_b2 = (float)(1.0 - (double)beta2);
+  a.step_size = (float)((double)lr / bc1);
+  a.bc2_sqrt = (float)sqrt(bc2);
+  a.eps = eps;
+  a.grad_scale = grad_scale;
+  return a;
+}
+
 int stream_grid(int64_t nvec) {
   // enough blocks to keep every CU busy with several waves, capped so that the grid-stride
   // loop amortises the launch
@@ -345,18 +447,7 @@ int pk_adamw_fused(float* master, float* exp_avg, float* exp_avg_sq, float* grad
   if (!pk_aligned16(master) || !pk_aligned16(exp_avg) || !pk_aligned16(exp_avg_sq) ||
       !pk_aligned16(grad) || (shadow && !pk_aligned16(shadow)))
     return PK_ERR_ALIGN;
-  // scalar prologue in double, as torch does on the host (python floats)
-  const double bc1 = 1.0 - pow((double)beta1, (double)step);
-  const double bc2 = 1.0 - pow((double)beta2, (double)step);
-  AdamArgs a;
-  a.decay = (float)(1.0 - (double)lr * (double)weight_decay);
-  a.one_m_b1 = (float)(1.0 - (double)beta1);
-  a.beta2 = beta2;
-  a.one_m_b2 = (float)(1.0 - (double)beta2);
-  a.step_size = (float)((double)lr / bc1);
-  a.bc2_sqrt = (float)sqrt(bc2);
-  a.eps = eps;
-  a.grad_scale = grad_scale;
+  const AdamArgs a = make_adam_args(lr, beta1, beta2, eps, weight_decay, step, grad_scale);
   hipStream_t s = (hipStream_t)stream;
   const int64_t nblocks = pk_ceil_div((n >> 2) > 0 ? (n >> 2) : 1, kStreamThreads);
   if (nblocks > 0x7fffffffll) return PK_ERR_SHAPE;
@@ -373,6 +464,70 @@ int pk_adamw_fused(float* master, float* exp_avg, float* exp_avg_sq, float* grad
   }
 #undef PK_ADAM_LAUNCH
   PK_RETURN_IF_LAUNCH_FAILED();
+  return PK_OK;
+}
+
+int pk_adamw_fused_packed(float* master, float* exp_avg, float* exp_avg_sq, float* flat_grad,
+                          const void* const* grads, const int64_t* offsets, const int64_t* numels, int64_t n,
+                          int grad_dtype, void* shadow, int shadow_dtype, float lr, float beta1, float beta2,
+                          float eps, float weight_decay, int64_t step, float grad_scale, int zero_grad,
+                          pk_stream_t stream) {
+  if (n < 0 || step < 1 || !pk_dtype_ok(grad_dtype)) return PK_ERR_ARG;
+  if (n == 0) return PK_OK;
+  if (!master || !exp_avg || !exp_avg_sq || !grads || !offsets || !numels) return PK_ERR_ARG;
+  if (shadow && shadow_dtype != PK_BF16) return PK_ERR_UNSUPPORTED;
+  if (!pk_aligned16(master) || !pk_aligned16(exp_avg) || !pk_aligned16(exp_avg_sq) ||
+      (flat_grad && !pk_aligned16(flat_grad)) || (shadow && !pk_aligned16(shadow)))
+    return PK_ERR_ALIGN;
+  for (int64_t i = 0; i < n; ++i)
+    if (numels[i] < 0 || offsets[i] < 0) return PK_ERR_ARG;
+  const AdamArgs a = make_adam_args(lr, beta1, beta2, eps, weight_decay, step, grad_scale);
+  hipStream_t s = (hipStream_t)stream;
+  int64_t i = 0;
+  while (i < n) {
+    PackArgs pa;
+    pa.n = 0;
+    int64_t blocks = 0;
+    while (i < n && pa.n < kPackTensorsPerLaunch) {
+      if (numels[i] > 0) {      // a tensor without a gradient of its own is still stepped (decay, moments)
+        const int64_t nb = pk_ceil_div(numels[i], kAdamPackChunk);
+        if (blocks + nb > 0x7fffffff) break;
+        pa.src[pa.n] = grads[i];
+        pa.off[pa.n] = offsets[i];
+        pa.numel[pa.n] = numels[i];
+        pa.blk_start[pa.n] = (int32_t)blocks;
+        blocks += nb;
+        ++pa.n;
+      }
+      ++i;
+    }
+    if (pa.n == 0) {
+      if (i < n) return PK_ERR_SHAPE;
+      break;
+    }
+    pa.blk_start[pa.n] = (int32_t)blocks;
+    const dim3 grid((unsigned)blocks), block(kStreamThreads);
+#define PK_ADAMP(TG, SH, FL, ZE)                                                                               \
+  PK_LAUNCH_NOCHECK(pk_timing::K_ADAMW, s, (adamw_packed_kernel<TG, bf16_t, SH, FL, ZE>), grid, block, 0, s, pa, master, \
+                    exp_avg, exp_avg_sq, flat_grad, reinterpret_cast<bf16_t*>(shadow), a)
+#define PK_ADAMP_G(TG)                                                                       \
+  do {                                                                                       \
+    if (shadow) {                                                                            \
+      if (!flat_grad) PK_ADAMP(TG, true, false, false);                                      \
+      else if (zero_grad) PK_ADAMP(TG, true, true, true);                                    \
+      else PK_ADAMP(TG, true, true, false);                                                  \
+    } else {                                                                                 \
+      if (!flat_grad) PK_ADAMP(TG, false, false, false);                                     \
+      else if (zero_grad) PK_ADAMP(TG, false, true, true);                                   \
+      else PK_ADAMP(TG, false, true, false);                                                 \
+    }                                                                                        \
+  } while (0)
+    if (grad_dtype == PK_BF16) PK_ADAMP_G(bf16_t);
+    else PK_ADAMP_G(float);
+#undef PK_ADAMP_G
+#undef PK_ADAMP
+    PK_RETURN_IF_LAUNCH_FAILED();
+  }
   return PK_OK;
 }
 

@@ -131,6 +131,9 @@ class StageExecutor:
     compute_stream: torch.cuda.Stream | None = None
     pack_stream: torch.cuda.Stream | None = None
     loss_fn: Any = None
+    # the pack that follows a bucket's last backward of the iteration is folded into the optimizer
+    # step (ParamStorage.hold_param_grads / FusedAdamW.step_packed)
+    fuse_last_pack: bool = False
     _fwd: dict = field(default_factory=dict)
     _inp_grads: dict = field(default_factory=dict)
     _wgrad_queues: dict = field(default_factory=dict)
@@ -164,6 +167,11 @@ class StageExecutor:
         ubids = list(self.stages.buckets.keys())
         # which task gathers / frees a bucket's parameters and which one packs its gradients
         lifetimes = plan_zero_lifetimes(tasks)
+        last_pack = {}          # bucket -> index of the task whose gradients are the last ones packed
+        if self.fuse_last_pack:
+            for ti, task in enumerate(tasks):
+                if ti in lifetimes and lifetimes[ti].reduce_grads_after:
+                    last_pack[task.ubid] = ti
         for ti, task in enumerate(tasks):
             tt = task.type
             life = lifetimes.get(ti)
@@ -218,7 +226,7 @@ class StageExecutor:
                 if split:
                     self._wgrad_queues[(task.ubid, task.mb)] = queue
                 if life.reduce_grads_after:
-                    self._pack_after_backward(task.ubid, cs, ps, pack_events)
+                    self._pack_after_backward(task.ubid, cs, ps, pack_events, hold=last_pack.get(task.ubid) == ti)
                 if life.free_params_after:
                     self._free_params_after(task.ubid, cs)
             elif tt is TaskType.BWD_W:
@@ -226,7 +234,7 @@ class StageExecutor:
                 with torch.cuda.stream(cs):
                     queue.run()
                 if life.reduce_grads_after:
-                    self._pack_after_backward(task.ubid, cs, ps, pack_events)
+                    self._pack_after_backward(task.ubid, cs, ps, pack_events, hold=last_pack.get(task.ubid) == ti)
                 if life.free_params_after:
                     self._free_params_after(task.ubid, cs)
             elif tt is TaskType.UPD:
@@ -244,8 +252,13 @@ class StageExecutor:
         evt.record(cs)
         self.params.defer_free_full_params(ubid, evt)
 
-    def _pack_after_backward(self, ubid, cs, ps, pack_events: dict) -> None:
-        """Gradient pack on the second stream, ordered after the backward that produced the grads."""
+    def _pack_after_backward(self, ubid, cs, ps, pack_events: dict, hold: bool = False) -> None:
+        """Gradient pack on the second stream, ordered after the backward that produced the grads.
+        hold: these are the bucket's last gradients of the iteration and the optimizer step, which
+        runs on the compute stream, takes them as they are."""
+        if hold:
+            self.params.hold_param_grads(ubid, cs)
+            return
         if ps is not cs:
             evt = torch.cuda.Event()
             evt.record(cs)

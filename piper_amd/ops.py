@@ -443,3 +443,36 @@ def adamw_fused(master, exp_avg, exp_avg_sq, grad, *, step: int, lr: float, beta
     call("pk_adamw_fused", ptr(master), ptr(exp_avg), ptr(exp_avg_sq), ptr(grad), ptr(shadow),
          dtype_code(shadow.dtype) if shadow is not None else 0, n, float(lr), float(beta1), float(beta2), float(eps),
          float(weight_decay), int(step), float(grad_scale), int(bool(zero_grad)), current_stream(master.device))
+
+
+def adamw_fused_packed(master, exp_avg, exp_avg_sq, flat_grad, grads: Sequence[torch.Tensor | None], offsets: Sequence[int],
+                       numels: Sequence[int], *, step: int, lr: float, beta1: float, beta2: float, eps: float,
+                       weight_decay: float, shadow: torch.Tensor | None = None, grad_scale: float = 1.0,
+                       zero_grad: bool = False) -> None:
+    """AdamW over the tensors of a bucket with the last gradient pack folded in: the gradient of a
+    tensor is its slice of `flat_grad` (fp32, may be None) plus `grads[i]` (may be None), and the
+    result equals bucket_pack(accumulate=True) followed by adamw_fused bit for bit."""
+    require_gpu(master)
+    n = len(grads)
+    _check(len(offsets) == n and len(numels) == n, "adamw_fused_packed: one offset and element count per tensor")
+    total = master.numel()
+    for t in (master, exp_avg, exp_avg_sq):
+        _check(t.dtype == torch.float32 and t.numel() == total and t.is_contiguous(), "adamw_fused_packed: fp32 contiguous buffers of equal size")
+    if flat_grad is not None:
+        _check(flat_grad.dtype == torch.float32 and flat_grad.numel() == total and flat_grad.is_contiguous(), "adamw_fused_packed: flat_grad must match the bucket")
+    live = [g for g in grads if g is not None]
+    gdtype = live[0].dtype if live else torch.bfloat16
+    _check(all(g.dtype == gdtype for g in live), "adamw_fused_packed: gradients of one call must share a dtype")
+    for g, off, num in zip(grads, offsets, numels):
+        _check(off >= 0 and off + num <= total, "adamw_fused_packed: tensor outside the bucket")
+        _check(g is None or g.numel() == num, "adamw_fused_packed: gradient size differs from the tensor's")
+    if shadow is not None:
+        _check(shadow.dtype == torch.bfloat16 and shadow.numel() == total and shadow.is_contiguous(), "adamw_fused_packed: bf16 shadow of the bucket's size")
+    grads = [None if g is None else g.contiguous() for g in grads]
+    arr_p = _ptr_array(grads)
+    arr_o = (C.c_int64 * max(n, 1))(*offsets)
+    arr_n = (C.c_int64 * max(n, 1))(*numels)
+    call("pk_adamw_fused_packed", ptr(master), ptr(exp_avg), ptr(exp_avg_sq), ptr(flat_grad), arr_p, arr_o, arr_n, n,
+         dtype_code(gdtype), ptr(shadow), dtype_code(shadow.dtype) if shadow is not None else 0, float(lr), float(beta1),
+         float(beta2), float(eps), float(weight_decay), int(step), float(grad_scale), int(bool(zero_grad)),
+         current_stream(master.device))

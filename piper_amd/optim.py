@@ -58,3 +58,22 @@ class FusedAdamW(torch.optim.Optimizer):
                                 weight_decay=group["weight_decay"], shadow=shadow,
                                 zero_grad=self.zero_grad_in_step and owns_grad)
         return loss
+
+    @torch.no_grad()
+    def step_packed(self, p: torch.Tensor, grads, offsets, numels, flat_grad: torch.Tensor | None = None) -> None:
+        """One step for the flat parameter `p` (a bucket) whose last gradients have not been packed:
+        tensor i of the bucket (elements offsets[i] .. +numels[i]) has the gradient flat_grad[...] (what
+        earlier microbatches packed, optional) + grads[i] (optional).  Same result as packing
+        grads into flat_grad and calling step() with p.grad = flat_grad, in one launch that
+        neither writes nor re-reads the fp32 gradient bucket."""
+        group = next(g for g in self.param_groups if any(q is p for q in g["params"]))
+        if not p.is_contiguous():
+            raise RuntimeError("FusedAdamW needs contiguous parameters (flatten them into a bucket)")
+        st = self._init_state(p)
+        st["step"] += 1
+        b1, b2 = group["betas"]
+        shadow = None if p.dtype == torch.float32 else p.detach().reshape(-1)
+        ops.adamw_fused_packed(st["master"], st["exp_avg"], st["exp_avg_sq"], flat_grad, list(grads), list(offsets),
+                               list(numels), step=st["step"], lr=group["lr"], beta1=b1, beta2=b2, eps=group["eps"],
+                               weight_decay=group["weight_decay"], shadow=shadow,
+                               zero_grad=self.zero_grad_in_step and flat_grad is not None)

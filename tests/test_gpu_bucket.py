@@ -204,3 +204,55 @@ def test_timing_select_brackets_one_kernel_only(dev):
         _lib.timing_select(None)
         _lib.timing_enable(False)
         _lib.timing_collect()
+
+
+@pytest.mark.parametrize("grad_dtype,param_dtype", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32)])
+@pytest.mark.parametrize("earlier_microbatches", [0, 2])
+def test_adamw_with_the_last_pack_folded_in_is_bit_identical(dev, grad_dtype, param_dtype, earlier_microbatches):
+    """pk_adamw_fused_packed against pk_bucket_pack(accumulate) followed by pk_adamw_fused: master,
+    moments and the bf16 parameter bucket bit for bit, over tensors whose sizes are not multiples of
+    the vector width, a tensor without a gradient, and three steps."""
+    print(f"[case] adamw with folded pack {grad_dtype} earlier={earlier_microbatches}", flush=True)
+    shapes = [(3, 5), (8192,), (1,), (777, 13), (2, 8200), (64, 64), (1027,)]
+    numels = [math.prod(s) for s in shapes]
+    esize = 2 if param_dtype == torch.bfloat16 else 4
+    offs, total = ops.bucket_plan(numels, esize, 256)
+    gen = torch.Generator().manual_seed(7)
+    master0 = torch.zeros(total)
+    for o, n in zip(offs, numels):
+        master0[o:o + n] = torch.randn(n, generator=gen) * 0.02
+    hp = dict(lr=ADAMW["lr"], beta1=ADAMW["betas"][0], beta2=ADAMW["betas"][1], eps=ADAMW["eps"], weight_decay=ADAMW["weight_decay"])
+
+    def state():
+        m = master0.clone().to(dev)
+        sh = m.to(torch.bfloat16) if param_dtype == torch.bfloat16 else None
+        return m, torch.zeros_like(m), torch.zeros_like(m), sh
+
+    two, one = state(), state()
+    for step in range(1, 4):
+        flat_two = torch.zeros(total, device=dev)
+        flat_one = torch.zeros(total, device=dev)
+        for mb in range(earlier_microbatches):
+            gs = [t.to(dev) for t in _tensors(100 * step + mb, shapes, grad_dtype)]
+            ops.bucket_pack(gs, offs, flat_two, accumulate=True)
+            ops.bucket_pack(gs, offs, flat_one, accumulate=True)
+        last = [t.to(dev) for t in _tensors(100 * step + 50, shapes, grad_dtype)]
+        last[2] = None if step == 2 else last[2]              # a tensor without a gradient in the last microbatch
+        ops.bucket_pack(last, offs, flat_two, accumulate=True)
+        ops.adamw_fused(two[0], two[1], two[2], flat_two, step=step, shadow=two[3], **hp)
+        ops.adamw_fused_packed(one[0], one[1], one[2], flat_one if earlier_microbatches else None, last, offs, numels,
+                               step=step, shadow=one[3], **hp)
+        torch.cuda.synchronize()
+        for a, b, name in zip(two, one, ("master", "exp_avg", "exp_avg_sq", "bf16 parameters")):
+            if a is not None:
+                assert torch.equal(a, b), (step, name)
+    assert float(one[1].abs().max()) > 0
+    # and one step against the oracle: torch.optim.AdamW on the oracle's packed gradient (1e-6 as everywhere)
+    if earlier_microbatches == 0:
+        grads = _tensors(150, shapes, grad_dtype)
+        z = torch.zeros(total)
+        ref_m, _, _ = OB.adamw_step_torch(master0, OB.pack(torch.zeros(total), grads, offs), z, z, 1, ADAMW["lr"],
+                                          ADAMW["betas"], ADAMW["eps"], ADAMW["weight_decay"])
+        m1, v1, s1, sh1 = state()
+        ops.adamw_fused_packed(m1, v1, s1, None, [t.to(dev) for t in grads], offs, numels, step=1, shadow=sh1, **hp)
+        assert (m1.cpu() - ref_m).abs().max().item() <= ADAMW_TOL

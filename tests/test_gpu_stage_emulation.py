@@ -286,3 +286,35 @@ def test_full_size_stage_properties(dev):
     for li in (0, 1):
         g = _packed_grad(index, li, "w2")
         assert int((g.abs().amax(dim=(1, 2)) > 0).sum()) == cfg[4]
+
+
+def test_last_pack_folded_into_the_optimizer_step(dev):
+    """StageExecutor(fuse_last_pack=True): the pack after a bucket's last backward is skipped and the
+    optimizer kernel reads those gradients directly.  Same updated parameters, bit for bit, as the
+    iteration that packs every microbatch."""
+    cfg, bucket_mb, _ = REDUCED["three_buckets"]
+    B, S, MB = 2, 64, 3
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(44)
+    shapes = _layer_shapes(*cfg[:6])
+    layers = [_init_layer(gen, shapes, dtype) for _ in range(2)]
+    xs = [torch.randn(B, S, cfg[0], generator=gen).to(dtype).to(dev) for _ in range(MB)]
+    results = {}
+    for fuse in (False, True):
+        print(f"[case] stage with fuse_last_pack={fuse}", flush=True)
+        store, ex, tasks, index, _ = _build(layers, cfg, dev, dtype, MB, bucket_mb)
+        ex.fuse_last_pack = fuse
+        with torch.nn.attention.sdpa_kernel(torch.nn.attention.SDPBackend.MATH):
+            out = ex.run(tasks, xs)
+            torch.cuda.synchronize()
+        params = {key: index[key][0].flat_params[index[key][1]:index[key][1] + index[key][2]].clone() for key in index}
+        masters = {key: index[key][0].shard_optimizer.state[index[key][0].shard_param]["master"][
+            index[key][1]:index[key][1] + index[key][2]].clone() for key in index}
+        results[fuse] = (torch.stack(out["losses"]), params, masters)
+        for b in store.buckets.values():
+            for st in b.with_companions():
+                assert st.pending_grads is None and all(p.grad is None for p, *_ in st.param_view_specs)
+    assert torch.equal(results[False][0], results[True][0])
+    for key in results[False][1]:
+        assert torch.equal(results[False][1][key], results[True][1][key]), ("parameter", key)
+        assert torch.equal(results[False][2][key], results[True][2][key]), ("master", key)
