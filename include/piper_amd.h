@@ -287,6 +287,10 @@ PK_API int pk_grouped_swiglu_wgrad_scaled(const void* d_out, const void* hs, con
  *   between experts are neither written nor read.
  * ldt >= pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype) and a multiple of 64; that query returns
  * 0 when the shape or dtype has no such path (use the entry points above then).
+ * d_g and d_u (the row-major outputs) may both be NULL in pk_grouped_swiglu_dgrad_dh_scaled_t: they
+ * are then not written, and pk_grouped_swiglu_dgrad_dx_t computes d_x_sorted = d_g . w1[e] + d_u . w3[e]
+ * (the second half of the input gradient, as pk_grouped_swiglu_dgrad_dx) from the transposed copies,
+ * so that the SwiGLU backward stores each of d_g, d_u once instead of twice.
  * pk_grouped_swiglu_wgrad_scaled_t computes the same d_w1, d_w2, d_w3 as
  * pk_grouped_swiglu_wgrad_scaled from d_out, x (through row_map / row_map_div) and the transposed
  * copies.  Both replace the autograd of qwen3_bmm_experts_patch.py:39-41 like the pair above.
@@ -303,6 +307,13 @@ PK_API int pk_grouped_swiglu_dgrad_dh_scaled_t(const void* d_out, const int32_t*
                                         void* d_gT, void* d_uT, void* hsT, int64_t ldt, float* d_scores,
                                         void* workspace, int64_t workspace_bytes, int64_t A, int64_t H,
                                         int64_t I, int64_t E, int dtype, pk_stream_t stream);
+/* HOST, tuning hint: 1 when leaving out the row-major d_g / d_u and running
+ * pk_grouped_swiglu_dgrad_dx_t is the faster pair for this shape (long experts), 0 when the
+ * row-major pair is (or the shape has no transposed path). */
+PK_API int pk_grouped_swiglu_dx_from_transposed_pays(int64_t A, int64_t H, int64_t I, int64_t E, int dtype);
+PK_API int pk_grouped_swiglu_dgrad_dx_t(const void* d_gT, const void* d_uT, int64_t ldt, const void* w1, const void* w3,
+                                 const int32_t* starts, void* d_x_sorted, int64_t A, int64_t H, int64_t I,
+                                 int64_t E, int dtype, pk_stream_t stream);
 PK_API int pk_grouped_swiglu_wgrad_scaled_t(const void* d_out, const void* hsT, const void* d_gT, const void* d_uT,
                                      int64_t ldt, const void* x, const int32_t* row_map, int64_t row_map_div,
                                      const int32_t* starts, const int32_t* expert_order, void* d_w1,

@@ -63,6 +63,8 @@ SIGNATURES = {
     # d_out row_map div scores w2 g u starts d_g d_u d_gT d_uT hsT ldt d_scores ws ws_bytes A H I E dtype stream
     "pk_grouped_swiglu_dgrad_dh_scaled_t": (_c_int, [_p, _p, _c_i64, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _c_i64, _p,
                                                      _p, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
+    "pk_grouped_swiglu_dx_from_transposed_pays": (_c_int, [_c_i64, _c_i64, _c_i64, _c_i64, _c_int]),
+    "pk_grouped_swiglu_dgrad_dx_t": (_c_int, [_p, _p, _c_i64, _p, _p, _p, _p, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),
     # d_out hsT d_gT d_uT ldt x row_map div starts order d_w1 d_w2 d_w3 accumulate A H I E dtype stream
     "pk_grouped_swiglu_wgrad_scaled_t": (_c_int, [_p, _p, _p, _p, _c_i64, _p, _p, _c_i64, _p, _p, _p, _p, _p, _c_int,
                                                   _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _p]),

@@ -676,7 +676,10 @@ __device__ __forceinline__ void mma_ktile(const char* At, const char* Bt, const 
 // lookups included) are resolved with scalar loads during the current k-loop.
 // EPI_SWIGLU: the BN tile rows are [32 gate | 32 up | 32 gate | 32 up ...] of BN/2 output
 // columns, so that a lane holds the gate and the up value of the same element.
-template <int BM, int BN, int BK, int WMW, int WNW, int NS, bool B_KC, int EPI>
+// A_T: the A operand comes from a transposed copy in blocks of 32 padded rows ([rows / 32][lda][32],
+// see padded_start): a k-tile of it is one run of consecutive memory per 32-row block, it sits in LDS
+// as [BK k][BM rows] and its fragments come out of the transposing LDS read.
+template <int BM, int BN, int BK, int WMW, int WNW, int NS, bool B_KC, int EPI, bool A_T = false>
 __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMParams p) {
   constexpr int NW = WMW * WNW, NTHREADS = 64 * NW;
   constexpr int WTM = BM / WMW, WTN = BN / WNW;          // wave tile
@@ -712,6 +715,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES + RM_BYTES + BOX_BYTES];
   constexpr int CPR = BK / 8, RPI = 64 / CPR;            // 16-byte chunks per A row, A rows per dma16
   static_assert(LA * RPI <= 64, "a wave's A rows of a tile: one entry per lane");
+  static_assert(!A_T || BM % 32 == 0, "whole 32-row blocks of the transposed copy");
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -764,7 +768,8 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
   const int kt_per_seg = p.Kseg / BK;
   const int nkt = kt_per_seg * p.nseg;
   const uint32_t row_bytes = (uint32_t)p.lda * 2u;
-  const uint32_t step_a = BK * 2, step_b = B_KC ? (uint32_t)(BK * 2) : (uint32_t)BK * (uint32_t)p.ldb * 2u;
+  // bytes from one k-tile of A to the next: BK elements of a row, or BK columns of a 32-row block
+  const uint32_t step_a = A_T ? BK * 64 : BK * 2, step_b = B_KC ? (uint32_t)(BK * 2) : (uint32_t)BK * (uint32_t)p.ldb * 2u;
 
   struct Unit {
     int row0, rows, nt;
@@ -783,12 +788,27 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     t.nt = __builtin_amdgcn_readfirstlane(nt);
     t.tcol = __builtin_amdgcn_readfirstlane(padded_start(s0, e) + mt * BM);
     t.b_base = uniform_i64(((int64_t)e * p.strideB + (B_KC ? (int64_t)nt * BN_OUT * p.ldb : (int64_t)nt * BN)) * 2);
-    t.a_base = p.row_map ? (int64_t)0 : uniform_i64((int64_t)t.row0 * p.lda * 2);
-    if (!p.row_map) {
+    if constexpr (A_T) {
+      // the unit's first row sits at padded row tcol (a multiple of 64): block tcol / 32, and block b of
+      // the copy starts at b * lda * 32 elements.  A lane's 16 bytes are 8 consecutive rows of one
+      // column; blocks past the unit's last row are read from its last block instead (valid memory,
+      // rows that are never stored).
+      t.a_base = uniform_i64((int64_t)(t.tcol >> 5) * p.lda * 64);
 #pragma unroll
       for (int i = 0; i < LA; ++i) {
-        const int rbase = (wave * LA + i) * RPI;     // first tile row of this dma16 (wave-uniform)
-        t.voff_a[i] = (uint32_t)min(rbase + lane / CPR, t.rows - 1) * row_bytes + a_kofs[i];   // rows past the range are never stored
+        int krow, cofs;
+        mn_slot<BM>(wave * LA + i, lane, krow, cofs);
+        const int blk = min(cofs >> 5, (t.rows - 1) >> 5);
+        t.voff_a[i] = (uint32_t)((blk * (int)p.lda + krow) * 32 + (cofs & 31)) * 2u;
+      }
+    } else {
+      t.a_base = p.row_map ? (int64_t)0 : uniform_i64((int64_t)t.row0 * p.lda * 2);
+      if (!p.row_map) {
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+          const int rbase = (wave * LA + i) * RPI;     // first tile row of this dma16 (wave-uniform)
+          t.voff_a[i] = (uint32_t)min(rbase + lane / CPR, t.rows - 1) * row_bytes + a_kofs[i];   // rows past the range are never stored
+        }
       }
     }
   };
@@ -953,7 +973,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
         if (wave_has_rows) {
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks)
-            load_frags<BK, TM, TN, true, B_KC, BM, BN>(fr[ks], st, st + A_BYTES, wm * WTM, wn * WTN, ks, lane);
+            load_frags<BK, TM, TN, !A_T, B_KC, BM, BN>(fr[ks], st, st + A_BYTES, wm * WTM, wn * WTN, ks, lane);
         }
         __builtin_amdgcn_sched_barrier(0);
         static_for<L>([&](auto pc) { issue_piece(pc); });
@@ -990,7 +1010,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
     } else {
       Frags<TM, TN> f0;     // fragments of the first k-step of the coming k-tile, read one tile ahead
       if (wave_has_rows)
-        load_frags<BK, TM, TN, true, B_KC, BM, BN>(f0, smem + cur * STAGE, smem + cur * STAGE + A_BYTES, wm * WTM, wn * WTN, 0, lane);
+        load_frags<BK, TM, TN, !A_T, B_KC, BM, BN>(f0, smem + cur * STAGE, smem + cur * STAGE + A_BYTES, wm * WTM, wn * WTN, 0, lane);
 
       // k-tile kt+1 has to be in LDS before the MFMAs of k-tile kt: its first fragments are read
       // while they run, so that no wave waits for LDS behind the barrier of the next tile
@@ -1002,7 +1022,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void ragged_m_kernel(const RaggedMP
         const char* st = smem + cur * STAGE;
         const char* stn = smem + (cur + 1 == NS ? 0 : cur + 1) * STAGE;
         if (wave_has_rows) {
-          mma_ktile<BK, TM, TN, true, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN, f0, acc,
+          mma_ktile<BK, TM, TN, !A_T, B_KC, BM, BN, L>(st, st + A_BYTES, stn, stn + A_BYTES, wm * WTM, wn * WTN, f0, acc,
                                                        [&](auto pc) {
                                                          issue_piece(pc);
                                                          if constexpr (decltype(pc)::value == L - 1) ld_advance();
@@ -2035,7 +2055,7 @@ inline SchedSlot* sched_slot_for_launch(hipStream_t s) {
   return base + sched_slot_index(dev, (const void*)s, capture, thread);
 }
 
-template <int BM, int BN, int BK, int WMW, int WNW, int NS, bool B_KC, int EPI>
+template <int BM, int BN, int BK, int WMW, int WNW, int NS, bool B_KC, int EPI, bool A_T = false>
 int launch_ragged_m(RaggedMParams p, int64_t A_rows, int kernel_id, hipStream_t s) {
   const int64_t max_units = (pk_ceil_div(A_rows, BM) + p.E) * p.n_tiles;
   if (max_units > 0x7ffffff0ll || p.ldb * (int64_t)(BN > BK ? BN : BK) * 2 > 0x7fffffffll) return PK_ERR_SHAPE;
@@ -2043,11 +2063,12 @@ int launch_ragged_m(RaggedMParams p, int64_t A_rows, int kernel_id, hipStream_t 
   // map, from the operand's first row with one (all the rows that the map can name: under 4 GiB)
   const int64_t a_span_rows = p.row_map ? pk_ceil_div(A_rows, p.map_div.d) : (int64_t)BM;
   if (p.lda * 2 > 0x7fffffffll || (a_span_rows + 1) * p.lda * 2 > 0xffffffffll) return PK_ERR_SHAPE;
+  if (A_T && p.row_map) return PK_ERR_ARG;
   if ((int64_t)p.Kseg * p.nseg < 2 * BK) return PK_ERR_SHAPE;
   const int64_t grid = max_units < persistent_grid() ? round_up_xcd(max_units) : persistent_grid();
   p.sched = sched_slot_for_launch(s);
   if (!p.sched) return PK_ERR_UNSUPPORTED;
-  PK_LAUNCH_NOCHECK(kernel_id, s, (ragged_m_kernel<BM, BN, BK, WMW, WNW, NS, B_KC, EPI>),
+  PK_LAUNCH_NOCHECK(kernel_id, s, (ragged_m_kernel<BM, BN, BK, WMW, WNW, NS, B_KC, EPI, A_T>),
                     dim3((unsigned)grid), dim3(64 * WMW * WNW), 0, s, p);
   PK_RETURN_IF_LAUNCH_FAILED();
   return PK_OK;
@@ -2183,7 +2204,7 @@ bool mfma_shape_ok(int64_t H, int64_t I) { return H % 128 == 0 && I % 128 == 0; 
 
 // Pick the tile width by the output width N of the GEMM (for the gate/up kernel a tile holds
 // BN/2 gate and BN/2 up columns).
-template <bool B_KC, int EPI>
+template <bool B_KC, int EPI, bool A_T = false>
 int launch_rm(mf::RaggedMParams& p, int64_t A, int64_t N, int kernel_id, hipStream_t s) {
   const int64_t per_tile_big = (EPI == mf::EPI_SWIGLU) ? PK_RM_BN / 2 : PK_RM_BN;
   if (N % per_tile_big == 0) {
@@ -2197,9 +2218,10 @@ int launch_rm(mf::RaggedMParams& p, int64_t A, int64_t N, int kernel_id, hipStre
     // 128 accumulator registers that epilogue spills (measured 14 % slower at 16,384 tokens even
     // with the packed outputs staged 32 columns at a time)
     if (EPI == mf::EPI_SWIGLU_BWD_SCALED || lowm || A < (int64_t)PK_RM_SHORT_ROWS * p.E)
-      return mf::launch_ragged_m<PK_RM_SHORT, B_KC, EPI>(p, A, kernel_id, s);
-    if constexpr (EPI != mf::EPI_SWIGLU_BWD_SCALED) return mf::launch_ragged_m<PK_RM_CFG, B_KC, EPI>(p, A, kernel_id, s);
+      return mf::launch_ragged_m<PK_RM_SHORT, B_KC, EPI, A_T>(p, A, kernel_id, s);
+    if constexpr (EPI != mf::EPI_SWIGLU_BWD_SCALED) return mf::launch_ragged_m<PK_RM_CFG, B_KC, EPI, A_T>(p, A, kernel_id, s);
   }
+  if constexpr (A_T) return PK_ERR_SHAPE;      // the transposed copies exist for widths that are multiples of 256 only
   const int64_t per_tile_alt = (EPI == mf::EPI_SWIGLU) ? 64 : 128;
   p.n_tiles = (int32_t)(N / per_tile_alt);
   return mf::launch_ragged_m<PK_RM_ALT, B_KC, EPI>(p, A, kernel_id, s);
@@ -2361,9 +2383,10 @@ static int dgrad_dh_scaled_impl(const void* d_out, const int32_t* row_map, int64
   if (rc) return rc;
   if (A == 0) return PK_OK;
   const bool transposed = d_gT != nullptr;
-  if (!d_out || !row_map || row_map_div <= 0 || row_map_div > 0x7fffffffll || !scores || !w2 || !g || !u || !starts || !d_g || !d_u || !d_scores)
+  if (!d_out || !row_map || row_map_div <= 0 || row_map_div > 0x7fffffffll || !scores || !w2 || !g || !u || !starts || !d_scores)
     return PK_ERR_ARG;
-  if (!hs && !transposed) return PK_ERR_ARG;
+  if ((!hs || !d_g || !d_u) && !transposed) return PK_ERR_ARG;      // the row-major outputs are optional beside the transposed ones
+  if ((d_g == nullptr) != (d_u == nullptr)) return PK_ERR_ARG;
   if (transposed) {
     const int64_t need = pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype);
     if (need <= 0) return PK_ERR_SHAPE;
@@ -2455,6 +2478,34 @@ int pk_grouped_swiglu_dgrad_dx(const void* d_g, const void* d_u, const void* w1,
   q.starts = starts; q.E = (int32_t)E; q.Kseg = (int32_t)I; q.nseg = 2;
   q.O0 = (bf16_t*)d_x_sorted; q.ldc = H;
   return launch_rm<false, mf::EPI_PLAIN>(q, A, H, pk_timing::K_SWIGLU_DGRAD_DX, s);
+}
+
+int pk_grouped_swiglu_dx_from_transposed_pays(int64_t A, int64_t H, int64_t I, int64_t E, int dtype) {
+  if (pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype) <= 0) return 0;
+  // measured on MI355X (H 2048, I 768, 128 experts): with 1,024 rows per expert the SwiGLU backward is
+  // 9 % and the d_x GEMM 4 % faster without the row-major copies (256-row units, the A tile arrives
+  // as runs of 4 KB); with 256 rows per expert the d_x GEMM on 128-row units loses 6 %, more than
+  // the SwiGLU backward gains
+  return A >= (int64_t)PK_RM_SHORT_ROWS * E ? 1 : 0;
+}
+
+int pk_grouped_swiglu_dgrad_dx_t(const void* d_gT, const void* d_uT, int64_t ldt, const void* w1, const void* w3,
+                                 const int32_t* starts, void* d_x_sorted, int64_t A, int64_t H, int64_t I,
+                                 int64_t E, int dtype, pk_stream_t stream) {
+  int rc = check_common(A, H, I, E, dtype);
+  if (rc) return rc;
+  const int64_t need = pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype);
+  if (need <= 0) return PK_ERR_SHAPE;
+  if (A == 0) return PK_OK;
+  if (!d_gT || !d_uT || !w1 || !w3 || !starts || !d_x_sorted || ldt < need || ldt % 64 != 0) return PK_ERR_ARG;
+  if (!all_aligned16({d_gT, d_uT, w1, w3, d_x_sorted})) return PK_ERR_ALIGN;
+  // d_x = [d_g | d_u] . [w1[e] ; w3[e]] with the A operand read from the 32-row blocks
+  mf::RaggedMParams q = {};
+  q.A0 = (const bf16_t*)d_gT; q.A1 = (const bf16_t*)d_uT; q.lda = I;
+  q.B0 = (const bf16_t*)w1; q.B1 = (const bf16_t*)w3; q.ldb = H; q.strideB = I * H;
+  q.starts = starts; q.E = (int32_t)E; q.Kseg = (int32_t)I; q.nseg = 2;
+  q.O0 = (bf16_t*)d_x_sorted; q.ldc = H;
+  return launch_rm<false, mf::EPI_PLAIN, true>(q, A, H, pk_timing::K_SWIGLU_DGRAD_DX, (hipStream_t)stream);
 }
 
 int pk_grouped_swiglu_dgrad(const void* d_y, const void* w1, const void* w2, const void* w3,

@@ -409,8 +409,18 @@ class _ExpertRegionFn(torch.autograd.Function):
         # shapes with a K-contiguous weight-gradient path get d_g, d_u and score*h transposed as well
         # (score*h only transposed): wgrad(...) below hides which of the two kernel pairs runs
         if ops.transposed_ld(perm.numel(), x.shape[1], g.shape[1], E, g.dtype) > 0:
-            d_g, d_u, d_gT, d_uT, hsT, d_scores = ops.grouped_swiglu_dgrad_dh_scaled_t(d_out, perm, top_scores, w2, g, u, starts)
+            # With long experts d_g and d_u exist only as the transposed copies: the weight gradient
+            # wants them that way, and the d_x GEMM reads its A operand from the same blocks.  With
+            # short experts the row-major pair for the d_x GEMM is written as well.
+            blocks_only = ops.dx_from_transposed_pays(perm.numel(), x.shape[1], g.shape[1], E, g.dtype)
+            d_g, d_u, d_gT, d_uT, hsT, d_scores = ops.grouped_swiglu_dgrad_dh_scaled_t(d_out, perm, top_scores, w2, g, u, starts,
+                                                                                       row_major=not blocks_only)
             h = None
+
+            def input_grad():
+                if blocks_only:
+                    return ops.grouped_swiglu_dgrad_dx_t(d_gT, d_uT, w1, w3, starts, perm.numel())
+                return ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
 
             def wgrad(**kw):
                 return ops.grouped_swiglu_wgrad_scaled_t(d_out, hsT, d_gT, d_uT, x, starts, E, row_map=perm,
@@ -418,6 +428,9 @@ class _ExpertRegionFn(torch.autograd.Function):
             wgrad_inputs = (d_out, hsT, d_gT, d_uT)
         else:
             d_g, d_u, h, d_scores = ops.grouped_swiglu_dgrad_dh_scaled(d_out, perm, top_scores, w2, g, u, starts)
+
+            def input_grad():
+                return ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
 
             def wgrad(**kw):
                 return ops.grouped_swiglu_wgrad(d_y, h, d_g, d_u, x, starts, E, row_map=perm, row_map_div=top_k,
@@ -433,7 +446,7 @@ class _ExpertRegionFn(torch.autograd.Function):
             # queued with the tensors they need and computed by the weight pass
             p_gate, p_bias = ctx.params[0], ctx.params[1]
             _queue_wgrad(ctx.params[2:], wgrad)
-            d_xs = ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
+            d_xs = input_grad()
             d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
             d_x32 = ops.gate_logits_bwd(d_logits, x, w_gate, need_dx=need[0], d_w_gate=None, d_gate_bias=None)
             d_x = ops.permute_bwd(d_xs, inv_perm, top_k, addend_f32=d_x32) if need[0] else None
@@ -459,7 +472,7 @@ class _ExpertRegionFn(torch.autograd.Function):
                     d_w1, d_w2, d_w3 = wgrad()
             else:
                 d_w1, d_w2, d_w3 = wgrad()
-        d_xs = ops.grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts)
+        d_xs = input_grad()
         d_logits = ops.route_topk_bwd(logits, top_idx, d_scores, route_norm, route_scale)
         if gate_in_place:
             d_wg = d_b = None

@@ -293,11 +293,13 @@ def transposed_ld(A: int, H: int, I: int, E: int, dtype: torch.dtype) -> int:
     return int(_lib.load().pk_grouped_swiglu_transposed_ld(A, H, I, E, dtype_code(dtype)))
 
 
-def grouped_swiglu_dgrad_dh_scaled_t(d_out, perm, top_scores, w2, g, u, starts):
+def grouped_swiglu_dgrad_dh_scaled_t(d_out, perm, top_scores, w2, g, u, starts, row_major: bool = True):
     """grouped_swiglu_dgrad_dh_scaled with the outputs the weight gradient reads written transposed:
     returns (d_g, d_u [A,I], d_gT, d_uT, hsT [ldt/32, I, 32], d_scores [T,K] f32).  A transposed copy
     holds, for every block of 32 padded rows, the I columns with the block's 32 row values
-    contiguous: element (column i, padded row r) sits at [r // 32, i, r % 32]."""
+    contiguous: element (column i, padded row r) sits at [r // 32, i, r % 32].  row_major=False:
+    d_g and d_u are not written (None is returned for them); grouped_swiglu_dgrad_dx_t then takes
+    the input gradient from the transposed copies."""
     require_gpu(d_out)
     E, H, I = w2.shape
     A = perm.numel()
@@ -305,8 +307,8 @@ def grouped_swiglu_dgrad_dh_scaled_t(d_out, perm, top_scores, w2, g, u, starts):
     dev = d_out.device
     ldt = transposed_ld(A, H, I, E, g.dtype)
     _check(ldt > 0, "grouped_swiglu_dgrad_dh_scaled_t: shape without a transposed path")
-    d_g = torch.empty_like(g)
-    d_u = torch.empty_like(u)
+    d_g = torch.empty_like(g) if row_major else None
+    d_u = torch.empty_like(u) if row_major else None
     d_gT, d_uT, hsT = (torch.empty((ldt // 32, I, 32), dtype=g.dtype, device=dev) for _ in range(3))
     d_scores = torch.empty((T, K), dtype=torch.float32, device=dev)
     ws_bytes = int(_lib.load().pk_grouped_swiglu_dgrad_dh_scaled_workspace_bytes(A, I))
@@ -334,6 +336,27 @@ def grouped_swiglu_wgrad_scaled_t(d_out, hsT, d_gT, d_uT, x, starts, E, *, row_m
          ptr(row_map), row_map_div, ptr(starts), ptr(expert_order), ptr(d_w1), ptr(d_w2), ptr(d_w3), int(bool(accumulate)),
          A, H, I, E, dtype_code(dt), current_stream(dev))
     return d_w1, d_w2, d_w3
+
+
+def dx_from_transposed_pays(A: int, H: int, I: int, E: int, dtype: torch.dtype) -> bool:
+    """Whether the fused backward should leave out the row-major d_g / d_u and take d_x from the
+    transposed copies (the library's own tuning hint)."""
+    if dtype not in (torch.float32, torch.bfloat16):
+        return False
+    return bool(_lib.load().pk_grouped_swiglu_dx_from_transposed_pays(A, H, I, E, dtype_code(dtype)))
+
+
+def grouped_swiglu_dgrad_dx_t(d_gT, d_uT, w1, w3, starts, num_rows: int):
+    """d_x_sorted [A,H] = d_g . w1 + d_u . w3 with d_g, d_u given as the transposed copies of
+    grouped_swiglu_dgrad_dh_scaled_t ([ldt/32, I, 32]); num_rows = A."""
+    require_gpu(d_gT)
+    E, I, H = w1.shape
+    ldt = d_gT.shape[0] * 32
+    _check(d_gT.shape == d_uT.shape and d_gT.shape[1] == I and d_gT.shape[2] == 32, "grouped_swiglu_dgrad_dx_t: [ldt/32, I, 32] copies")
+    d_x = torch.empty((num_rows, H), dtype=d_gT.dtype, device=d_gT.device)
+    call("pk_grouped_swiglu_dgrad_dx_t", ptr(d_gT), ptr(d_uT), ldt, ptr(w1.contiguous()), ptr(w3.contiguous()), ptr(starts),
+         ptr(d_x), num_rows, H, I, E, dtype_code(d_gT.dtype), current_stream(d_gT.device))
+    return d_x
 
 
 def grouped_swiglu_dgrad_dx(d_g, d_u, w1, w3, starts):

@@ -189,6 +189,9 @@ T_CASES = [
     ([3000, 0, 1, 2500, 33, 0, 700, 600, 500, 400, 300, 64, 32, 70, 100, 96], 1024, 768),
     # ... and the static hand-out with many short experts (reductions of 0 to 3 k-tiles back to back)
     ([0, 1, 33, 64, 5, 96, 31, 70, 0, 0, 65, 2] * 24, 256, 256),
+    # enough 256-row units per workgroup for the 256x256x32 tiles (the d_x GEMM then reads 32-deep
+    # k-tiles of the transposed copies), with ragged last row tiles
+    ([8192, 8000, 8300, 7777, 8192, 8448, 8193, 8190], 1024, 256),
 ]
 
 
@@ -234,6 +237,19 @@ def test_transposed_backward_pair_matches_the_plain_pair(dev, counts, H, I):
             blk = tr.permute(1, 0, 2).reshape(I, ldt)[:, p0:p0 + c32]
             assert torch.equal(blk[:, :c], full[st[e]:st[e] + c].t()), f"expert {e}"
             assert torch.count_nonzero(blk[:, c:]).item() == 0, f"pad columns of expert {e}"
+
+    # without the row-major outputs: the same transposed copies, and the d_x GEMM that reads its A
+    # operand from them gives the d_x of the row-major pair bit for bit (same products, same order)
+    none_g, none_u, d_gT3, d_uT3, hsT3, d_s3 = ops.grouped_swiglu_dgrad_dh_scaled_t(DO, PERM, SC, W2, g, u, starts, row_major=False)
+    assert none_g is None and none_u is None and torch.equal(d_s3, d_s)
+    for e, c in enumerate(counts):
+        p0 = (st[e] // 64) * 64 + 64 * e
+        c32 = (c + 31) // 32 * 32
+        for a, b in ((d_gT, d_gT3), (d_uT, d_uT3), (hsT, hsT3)):
+            assert torch.equal(a.permute(1, 0, 2).reshape(I, ldt)[:, p0:p0 + c32], b.permute(1, 0, 2).reshape(I, ldt)[:, p0:p0 + c32])
+    d_x_rows = ops.grouped_swiglu_dgrad_dx(d_g, d_u, W1, W3, starts)
+    d_x_blocks = ops.grouped_swiglu_dgrad_dx_t(d_gT3, d_uT3, W1, W3, starts, A)
+    assert torch.equal(d_x_rows, d_x_blocks)
 
     ref = ops.grouped_swiglu_wgrad(DO, hs, d_g, d_u, XT, starts, E, row_map=PERM, row_map_div=K, scaled=True)
     order = torch.argsort(cnt, descending=True, stable=True).to(torch.int32).to(dev)
