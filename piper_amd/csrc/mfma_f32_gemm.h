@@ -20,6 +20,7 @@ struct Params {
   int64_t sbk, sbn;    // element strides of B(k,n)
   int32_t splits;
   int32_t accumulate;  // splits == 1: C += result
+  int64_t plane_a, plane_b;   // elements between the bf16 planes of a pre-split operand (mfma_x3_gemm.h)
 };
 
 // Four consecutive elements of an operand as floats (16-byte / 8-byte load).

@@ -8,6 +8,10 @@
 // cycles.  Same Params, tiling, split-K and epilogue as mfma_f32_gemm.h.  An operand whose k index
 // is not the contiguous one is kept in LDS as [k][row] (8-byte stores of the 4 fetched elements)
 // and turned into MFMA fragments by the transposing LDS read (ds_read_b64_tr_b16).
+// An fp32 operand can also be handed over already split (split3_t: three bf16 planes in memory, made
+// once by split_planes_kernel): every workgroup that loads a tile of an fp32 operand otherwise
+// splits it again, and with tiles this small that arithmetic (about 20 vector instructions per
+// MFMA) is what the kernels spend most of their time on.
 #pragma once
 #include "mfma_f32_gemm.h"
 #include <type_traits>
@@ -38,9 +42,41 @@ __device__ __forceinline__ bf16x8_t frag_mn(const bf16_t* tile, int ld, int row0
   return __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 
+// operand element types: float (split on load), bf16_t (one plane), split3_t (three bf16 planes in
+// memory: plane q of element i at base[q * plane_stride + i])
+struct split3_t {};
 template <typename T> struct Planes;
 template <> struct Planes<float> { static constexpr int N = 3; };
 template <> struct Planes<bf16_t> { static constexpr int N = 1; };
+template <> struct Planes<split3_t> { static constexpr int N = 3; };
+template <typename T> struct Mem { typedef T type; };
+template <> struct Mem<split3_t> { typedef bf16_t type; };      // what the operand pointer points at
+
+// fp32 [n] -> three bf16 planes [3][n]: hi = bf16(v), mid = bf16(v - hi), lo = bf16(v - hi - mid)
+__global__ __launch_bounds__(256) void split_planes_kernel(const float* __restrict__ src, bf16_t* __restrict__ dst, int64_t n) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i + 4 <= n) {
+    const float4 v = *reinterpret_cast<const float4*>(src + i);
+    const float f[4] = {v.x, v.y, v.z, v.w};
+    bf16x4_t pl[3];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bf16_t hi = (bf16_t)f[j];
+      const float r1 = f[j] - (float)hi;
+      const bf16_t mid = (bf16_t)r1;
+      pl[0][j] = hi; pl[1][j] = mid; pl[2][j] = (bf16_t)(r1 - (float)mid);
+    }
+#pragma unroll
+    for (int q = 0; q < 3; ++q) *reinterpret_cast<bf16x4_t*>(dst + q * n + i) = pl[q];
+  } else {
+    for (int64_t e = i; e < n; ++e) {
+      const bf16_t hi = (bf16_t)src[e];
+      const float r1 = src[e] - (float)hi;
+      const bf16_t mid = (bf16_t)r1;
+      dst[e] = hi; dst[n + e] = mid; dst[2 * n + e] = (bf16_t)(r1 - (float)mid);
+    }
+  }
+}
 
 template <int P>
 __device__ __forceinline__ void split(float v, bf16_t (&out)[P]) {
@@ -49,6 +85,31 @@ __device__ __forceinline__ void split(float v, bf16_t (&out)[P]) {
     const float r1 = v - (float)out[0];
     out[1] = (bf16_t)r1;
     if (P > 2) out[2] = (bf16_t)(r1 - (float)out[1]);
+  }
+}
+template <int P>
+__device__ __forceinline__ void zero_planes(bf16x4_t (&out)[P]) {
+  const bf16x4_t zero = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+#pragma unroll
+  for (int q = 0; q < P; ++q) out[q] = zero;
+}
+// four consecutive elements of an operand as planes of four bf16
+template <typename T>
+__device__ __forceinline__ void fetch4(const typename Mem<T>::type* src, int64_t plane_stride, bf16x4_t (&out)[Planes<T>::N]) {
+  constexpr int P = Planes<T>::N;
+  if constexpr (std::is_same<T, float>::value) {
+    float v[4];
+    pk_f32mm::load4<float>(src, v);
+    bf16_t pl[4][P];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) split<P>(v[j], pl[j]);
+#pragma unroll
+    for (int q = 0; q < P; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) out[q][j] = pl[j][q];
+  } else {
+#pragma unroll
+    for (int q = 0; q < P; ++q) out[q] = *reinterpret_cast<const bf16x4_t*>(src + q * plane_stride);
   }
 }
 
@@ -67,18 +128,21 @@ __global__ __launch_bounds__(64 * WM * WN) void kernel(const Params p) {
   const int64_t kbeg = (int64_t)blockIdx.z * kchunk;
   const int64_t kend = kbeg + kchunk < p.K ? kbeg + kchunk : p.K;
 
-  const TA* A = reinterpret_cast<const TA*>(p.A);
-  const TB* B = reinterpret_cast<const TB*>(p.B);
+  typedef typename Mem<TA>::type MA;
+  typedef typename Mem<TB>::type MB;
+  const MA* A = reinterpret_cast<const MA*>(p.A);
+  const MB* B = reinterpret_cast<const MB*>(p.B);
 
   floatx16_t acc;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 
-  // every thread fetches 4 consecutive elements of the contiguous index per load; the loads of
-  // tile k+1 are in flight while tile k is multiplied
+  // every thread fetches 4 consecutive elements of the contiguous index per load (every plane of
+  // them for a pre-split operand); the loads of tile k+1 are in flight while tile k is multiplied
   constexpr int NA = BM * BK / (THREADS * 4), NB = BN * BK / (THREADS * 4);
   static_assert(NA >= 1 && NB >= 1, "tile too small for the thread count");
-  float ra[NA][4], rb[NB][4];
+  // four fetched elements as planes of four bf16 (an fp32 operand is split here, once per load)
+  bf16x4_t ra[NA][PA], rb[NB][PB];
   auto slot = [](int idx, bool kc, int R, int& row, int& k) {
     if (kc) { k = (idx % (BK / 4)) * 4; row = idx / (BK / 4); }
     else { row = (idx % (R / 4)) * 4; k = idx / (R / 4); }
@@ -88,35 +152,23 @@ __global__ __launch_bounds__(64 * WM * WN) void kernel(const Params p) {
     for (int i = 0; i < NA; ++i) {
       int m, k;
       slot(tid + i * THREADS, A_KC, BM, m, k);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) ra[i][j] = 0.f;
-      if (m0 + m < p.M && k0 + k < kend)
-        pk_f32mm::load4<TA>(A + (m0 + m) * p.sam + (k0 + k) * p.sak, ra[i]);
+      zero_planes<PA>(ra[i]);
+      if (m0 + m < p.M && k0 + k < kend) fetch4<TA>(A + (m0 + m) * p.sam + (k0 + k) * p.sak, p.plane_a, ra[i]);
     }
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       int n, k;
       slot(tid + i * THREADS, B_KC, BN, n, k);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) rb[i][j] = 0.f;
-      if (n0 + n < p.N && k0 + k < kend)
-        pk_f32mm::load4<TB>(B + (k0 + k) * p.sbk + (n0 + n) * p.sbn, rb[i]);
+      zero_planes<PB>(rb[i]);
+      if (n0 + n < p.N && k0 + k < kend) fetch4<TB>(B + (k0 + k) * p.sbk + (n0 + n) * p.sbn, p.plane_b, rb[i]);
     }
   };
-  // split 4 fetched elements into planes; one 8-byte store per plane: along k of a [row][k] tile
-  // for a K-contiguous operand, along the rows of a [k][row] tile otherwise
-  auto store4 = [](auto& tiles, auto nplanes, bool kc, int ld_mn, int row, int k, const float (&v)[4]) {
+  // one 8-byte store per plane: along k of a [row][k] tile for a K-contiguous operand, along the
+  // rows of a [k][row] tile otherwise
+  auto store4 = [](auto& tiles, auto nplanes, bool kc, int ld_mn, int row, int k, const auto& v) {
     constexpr int P = decltype(nplanes)::value;
-    bf16_t pl[4][P];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) split<P>(v[j], pl[j]);
-#pragma unroll
-    for (int q = 0; q < P; ++q) {
-      bf16x4_t o;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) o[j] = pl[j][q];
-      *reinterpret_cast<bf16x4_t*>(&tiles[q][kc ? row * LDK + k : k * ld_mn + row]) = o;
-    }
+    for (int q = 0; q < P; ++q) *reinterpret_cast<bf16x4_t*>(&tiles[q][kc ? row * LDK + k : k * ld_mn + row]) = v[q];
   };
   if (kbeg < kend) load_tile(kbeg);
   for (int64_t k0 = kbeg; k0 < kend; k0 += BK) {
@@ -174,13 +226,20 @@ __global__ __launch_bounds__(64 * WM * WN) void kernel(const Params p) {
 template <int WM, int WN, bool A_KC, bool B_KC, typename TA, typename TB>
 inline bool usable(const Params& p) {
   using pk_f32mm::vec4_ok;
-  return (A_KC ? (p.sak == 1 && vec4_ok<TA>(p.A, p.K, p.sam)) : (p.sam == 1 && vec4_ok<TA>(p.A, p.M, p.sak))) &&
-         (B_KC ? (p.sbk == 1 && vec4_ok<TB>(p.B, p.K, p.sbn)) : (p.sbn == 1 && vec4_ok<TB>(p.B, p.N, p.sbk)));
+  typedef typename Mem<TA>::type MA;
+  typedef typename Mem<TB>::type MB;
+  if (std::is_same<TA, split3_t>::value && p.plane_a % 4 != 0) return false;
+  if (std::is_same<TB, split3_t>::value && p.plane_b % 4 != 0) return false;
+  return (A_KC ? (p.sak == 1 && vec4_ok<MA>(p.A, p.K, p.sam)) : (p.sam == 1 && vec4_ok<MA>(p.A, p.M, p.sak))) &&
+         (B_KC ? (p.sbk == 1 && vec4_ok<MB>(p.B, p.K, p.sbn)) : (p.sbn == 1 && vec4_ok<MB>(p.B, p.N, p.sbk)));
 }
 
 template <int WM, int WN, bool A_KC, bool B_KC, typename TA, typename TB>
 inline int launch(const Params& p, int kernel_id, hipStream_t s) {
-  if (!usable<WM, WN, A_KC, B_KC, TA, TB>(p)) return pk_f32mm::launch<WM, WN, A_KC, B_KC, TA, TB>(p, kernel_id, s);
+  if (!usable<WM, WN, A_KC, B_KC, TA, TB>(p)) {
+    if constexpr (std::is_same<TA, split3_t>::value || std::is_same<TB, split3_t>::value) return PK_ERR_ALIGN;   // the caller splits only what this kernel can read
+    else return pk_f32mm::launch<WM, WN, A_KC, B_KC, TA, TB>(p, kernel_id, s);
+  }
   if (p.M <= 0 || p.N <= 0) return PK_OK;
   dim3 grid((unsigned)pk_ceil_div(p.N, 32 * WN), (unsigned)pk_ceil_div(p.M, 32 * WM), (unsigned)p.splits);
   if (grid.y > 65535u || grid.z > 65535u) return PK_ERR_SHAPE;

@@ -407,10 +407,24 @@ static int gate_fwd_splits(int64_t H) {
   return (int)(sp < 1 ? 1 : (sp > 8 ? 8 : sp));
 }
 
-int64_t pk_gate_workspace_bytes(int64_t T, int64_t H, int64_t E) {
-  if (T < 0 || H <= 0 || E <= 0) return PK_ERR_ARG;
+static int64_t align256(int64_t n) { return (n + 255) / 256 * 256; }
+// bytes of the three bf16 planes of an fp32 array of n elements (0: cannot be pre-split)
+static int64_t plane_bytes(int64_t n) { return n % 4 == 0 ? align256(3 * n * (int64_t)sizeof(bf16_t)) : 0; }
+// fp32 [n] -> bf16 planes [3][n] at dst
+static int split_planes(const float* src, bf16_t* dst, int64_t n, int kernel_id, hipStream_t s) {
+  PK_LAUNCH_NOCHECK(kernel_id, s, pk_x3mm::split_planes_kernel, dim3((unsigned)pk_ceil_div(n, 1024)), dim3(256), 0, s, src, dst, n);
+  PK_RETURN_IF_LAUNCH_FAILED();
+  return PK_OK;
+}
+
+static int64_t gate_fwd_partial_bytes(int64_t T, int64_t H, int64_t E) {
   const int sp = gate_fwd_splits(H);
   return sp > 1 ? (int64_t)sp * T * E * (int64_t)sizeof(float) : 0;
+}
+
+int64_t pk_gate_workspace_bytes(int64_t T, int64_t H, int64_t E) {
+  if (T < 0 || H <= 0 || E <= 0) return PK_ERR_ARG;
+  return gate_fwd_partial_bytes(T, H, E);
 }
 
 int pk_gate_logits(const void* x, int x_dtype, const float* w_gate, const float* gate_bias,
@@ -425,7 +439,9 @@ int pk_gate_logits(const void* x, int x_dtype, const float* w_gate, const float*
   // writes and re-reads a [T, E] fp32 partial result, which soon outweighs reading x
   const int64_t row_tiles = pk_ceil_div(T, 64);
   while (sp > 1 && row_tiles * (sp / 2) >= 512) sp /= 2;
-  if (sp > 1 && (!workspace || workspace_bytes < pk_gate_workspace_bytes(T, H, E))) sp = 1;
+  if (sp > 1 && (!workspace || workspace_bytes < gate_fwd_partial_bytes(T, H, E))) sp = 1;
+  // (Handing this GEMM the weight already split into bf16 planes does not shorten it: the kernel
+  // waits on its loads and barriers, not on the instructions of the split.)
   pk_f32mm::Params p = {};
   p.A = x; p.B = w_gate;
   p.C = sp > 1 ? reinterpret_cast<float*>(workspace) : logits;
@@ -434,15 +450,13 @@ int pk_gate_logits(const void* x, int x_dtype, const float* w_gate, const float*
   p.sam = H; p.sak = 1; p.sbk = 1; p.sbn = H;
   p.splits = sp; p.accumulate = 0;
   int rc;
-  if (E > 64) {  // 64-token x 128-expert tiles, 8 waves
-    rc = x_dtype == PK_BF16
-             ? pk_x3mm::launch<2, 4, true, true, bf16_t, float>(p, pk_timing::K_GATE_LOGITS, s)
-             : pk_x3mm::launch<2, 4, true, true, float, float>(p, pk_timing::K_GATE_LOGITS, s);
-  } else {       // 64-token x 64-expert tiles, 4 waves
-    rc = x_dtype == PK_BF16
-             ? pk_x3mm::launch<2, 2, true, true, bf16_t, float>(p, pk_timing::K_GATE_LOGITS, s)
-             : pk_x3mm::launch<2, 2, true, true, float, float>(p, pk_timing::K_GATE_LOGITS, s);
-  }
+  const bool xb = x_dtype == PK_BF16;
+  if (E > 64)  // 64-token x 128-expert tiles, 8 waves
+    rc = xb ? pk_x3mm::launch<2, 4, true, true, bf16_t, float>(p, pk_timing::K_GATE_LOGITS, s)
+            : pk_x3mm::launch<2, 4, true, true, float, float>(p, pk_timing::K_GATE_LOGITS, s);
+  else         // 64-token x 64-expert tiles, 4 waves
+    rc = xb ? pk_x3mm::launch<2, 2, true, true, bf16_t, float>(p, pk_timing::K_GATE_LOGITS, s)
+            : pk_x3mm::launch<2, 2, true, true, float, float>(p, pk_timing::K_GATE_LOGITS, s);
   if (rc != PK_OK) return rc;
   if (sp > 1) {
     const int64_t n = T * E;
@@ -459,10 +473,18 @@ static int gate_bwd_splits(int64_t T) {
   return (int)(sp < 1 ? 1 : (sp > 16 ? 16 : sp));
 }
 
+// workspace of the backward: [split-K partials of d_w_gate, reused for the bias partial sums]
+// [d_logits as three bf16 planes, for the weight gradient]
+static int64_t gate_bwd_partial_bytes(int64_t T, int64_t H, int64_t E) {
+  const int sp = gate_bwd_splits(T);
+  const int64_t part = sp > 1 ? (int64_t)sp * E * H * (int64_t)sizeof(float) : 0;
+  const int64_t colsum = (int64_t)kColsumBlocks * E * (int64_t)sizeof(float);
+  return align256(part > colsum ? part : colsum);
+}
+
 int64_t pk_gate_bwd_workspace_bytes(int64_t T, int64_t H, int64_t E) {
   if (T < 0 || H <= 0 || E <= 0) return PK_ERR_ARG;
-  const int sp = gate_bwd_splits(T);
-  return sp > 1 ? (int64_t)sp * E * H * (int64_t)sizeof(float) : 0;
+  return gate_bwd_partial_bytes(T, H, E) + plane_bytes(T * E);
 }
 
 int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const float* w_gate,
@@ -472,6 +494,10 @@ int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const 
   if (T < 0 || H <= 0 || E <= 0 || !pk_dtype_ok(x_dtype)) return PK_ERR_ARG;
   if (!d_logits && T > 0) return PK_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
+  using pk_x3mm::split3_t;
+  const int64_t part_bytes = gate_bwd_partial_bytes(T, H, E);
+  const bool have_ws = workspace && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
+  const bool have_part = have_ws && workspace_bytes >= part_bytes;
   if (d_x_f32 && T > 0) {
     if (!w_gate) return PK_ERR_ARG;
     pk_f32mm::Params p = {};
@@ -485,16 +511,33 @@ int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const 
   if (d_w_gate) {
     if (!x && T > 0) return PK_ERR_ARG;
     int sp = gate_bwd_splits(T);
-    if (sp > 1 && (!workspace || workspace_bytes < pk_gate_bwd_workspace_bytes(T, H, E))) sp = 1;
+    if (sp > 1 && !have_part) sp = 1;
     pk_f32mm::Params p = {};
-    p.A = d_logits; p.B = x;
+    p.B = x;
     p.C = sp > 1 ? reinterpret_cast<float*>(workspace) : d_w_gate;
     p.M = E; p.N = H; p.K = T;
     p.sam = 1; p.sak = E; p.sbk = H; p.sbn = 1;
     p.splits = sp; p.accumulate = (sp == 1 && accumulate) ? 1 : 0;
-    int rc = x_dtype == PK_BF16
-                 ? pk_x3mm::launch<2, 2, false, false, float, bf16_t>(p, pk_timing::K_GATE_LOGITS_BWD, s)
-                 : pk_x3mm::launch<2, 2, false, false, float, float>(p, pk_timing::K_GATE_LOGITS_BWD, s);
+    // d_logits, whose every tile is read by H / 64 workgroups, is split into its three bf16 planes
+    // once when the workspace has room for them (this GEMM at 16,384 tokens: 74 -> 61 us, the split
+    // included); the kernel splits the tiles it loads otherwise
+    const int64_t pb = plane_bytes(T * E);
+    const bool presplit = T > 0 && have_ws && pb > 0 && E % 4 == 0 && workspace_bytes >= part_bytes + pb &&
+                          reinterpret_cast<uintptr_t>(d_logits) % 16 == 0;
+    int rc = PK_ERR_ALIGN;
+    if (presplit) {
+      bf16_t* planes = reinterpret_cast<bf16_t*>(reinterpret_cast<char*>(workspace) + part_bytes);
+      rc = split_planes(d_logits, planes, T * E, pk_timing::K_GATE_LOGITS_BWD, s);
+      if (rc != PK_OK) return rc;
+      p.A = planes; p.plane_a = T * E;
+      rc = x_dtype == PK_BF16 ? pk_x3mm::launch<2, 2, false, false, split3_t, bf16_t>(p, pk_timing::K_GATE_LOGITS_BWD, s)
+                              : pk_x3mm::launch<2, 2, false, false, split3_t, float>(p, pk_timing::K_GATE_LOGITS_BWD, s);
+    }
+    if (rc == PK_ERR_ALIGN) {  // no planes, or x cannot be read four elements at a time
+      p.A = d_logits;
+      rc = x_dtype == PK_BF16 ? pk_x3mm::launch<2, 2, false, false, float, bf16_t>(p, pk_timing::K_GATE_LOGITS_BWD, s)
+                              : pk_x3mm::launch<2, 2, false, false, float, float>(p, pk_timing::K_GATE_LOGITS_BWD, s);
+    }
     if (rc != PK_OK) return rc;
     if (sp > 1) {
       const int64_t n = E * H;
@@ -506,9 +549,9 @@ int pk_gate_logits_bwd(const float* d_logits, const void* x, int x_dtype, const 
     }
   }
   if (d_gate_bias) {
-    // (the workspace is free again here: the reduction above has consumed the GEMM's partial results)
-    const int64_t part_bytes = (int64_t)kColsumBlocks * E * (int64_t)sizeof(float);
-    if (T >= 32 * kColsumBlocks && E % 4 == 0 && E <= 1024 && workspace && workspace_bytes >= part_bytes &&
+    // (the first part of the workspace is free again here: the reduction above has consumed the GEMM's partial results)
+    const int64_t colsum_bytes = (int64_t)kColsumBlocks * E * (int64_t)sizeof(float);
+    if (T >= 32 * kColsumBlocks && E % 4 == 0 && E <= 1024 && workspace && workspace_bytes >= colsum_bytes &&
         reinterpret_cast<uintptr_t>(d_logits) % 16 == 0) {
       float* part = reinterpret_cast<float*>(workspace);
       PK_LAUNCH_NOCHECK(pk_timing::K_MISC, s, colsum_partial_kernel, dim3(kColsumBlocks), dim3(256), 0, s, d_logits, T,
