@@ -77,15 +77,31 @@ def kernel_bytes(cfg) -> dict:
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
 # counters read for a plain device copy of known size.  The numbers and the commands that produced
-# them are in the file named here; a kernel without a committed measurement reports null.
+# them are in the file named here, whose table this reads (first cell "<workload>:<kernel key>",
+# fifth and sixth cell read MB and written MB); a kernel without a row reports null.
 TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.md"
-MEASURED_TRAFFIC_BYTES = {      # (read + written) * 1e6, copied from that file
-    "cfg3": {"swiglu_gate_up": (1070 + 151) * 1e6, "swiglu_down": (483 + 134) * 1e6, "swiglu_dgrad_dh": (807 + 262) * 1e6,
-             "swiglu_dgrad_dx": (976 + 134) * 1e6, "swiglu_wgrad_w13": (355 + 807) * 1e6, "swiglu_wgrad_w2": (213 + 403) * 1e6},
-    "cfg4": {"swiglu_gate_up": (2745 + 606) * 1e6, "swiglu_down": (1292 + 537) * 1e6, "swiglu_dgrad_dh": (2179 + 1023) * 1e6,
-             "swiglu_dgrad_dx": (2612 + 537) * 1e6, "swiglu_wgrad_w13": (1626 + 806) * 1e6, "swiglu_wgrad_w2": (961 + 403) * 1e6},
-    "cfg2": {"pack+adamw": (334 + 680 + 2674 + 2378) * 1e6},
-}
+
+
+def measured_traffic_bytes() -> dict:
+    """{workload: {kernel key: (read + written) bytes per launch}} from the committed counter summary."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), TRAFFIC_SOURCE)
+    out: dict = {}
+    try:
+        with open(path) as f:
+            rows = [line.split("|") for line in f if line.startswith("| `")]
+    except OSError:
+        return out
+    for cells in rows:
+        try:
+            workload, key = cells[1].strip().strip("`").split(":")
+            read_mb, written_mb = (float(cells[i].replace(",", "")) for i in (5, 6))
+        except (ValueError, IndexError):
+            continue
+        out.setdefault(workload, {})[key] = (read_mb + written_mb) * 1e6
+    return out
+
+
+MEASURED_TRAFFIC_BYTES = measured_traffic_bytes()
 
 
 def bench_region(cfg, steps: int, warmup: int, accumulate: bool = False):
@@ -226,7 +242,8 @@ def bench_bucket(steps: int, warmup: int):
     pack_bytes = 6.0 * n_elems            # read bf16 grad, write fp32 bucket
     adam_bytes = 30.0 * total             # read g,p,m,v (16) + write p,m,v (12) + bf16 parameter (2)
     agg_gbs = (pack_bytes + adam_bytes) * steps / elapsed / 1e9
-    traffic = MEASURED_TRAFFIC_BYTES.get("cfg2", {}).get("pack+adamw")
+    cfg2_traffic = MEASURED_TRAFFIC_BYTES.get("cfg2", {})
+    traffic = cfg2_traffic["pack"] + cfg2_traffic["adamw"] if {"pack", "adamw"} <= set(cfg2_traffic) else None
     return {
         "metric": "bucket pack + fused AdamW HBM GB/s",
         "value": agg_gbs, "unit": "GB/s", "ms_per_step": elapsed / steps * 1e3,
@@ -246,6 +263,7 @@ def bench_bucket(steps: int, warmup: int):
         "fused_last_pack": {"ms_per_step": fused_elapsed / steps * 1e3, "bytes_per_element": 28,
                             "GB/s": 28.0 * n_elems * steps / fused_elapsed / 1e9,
                             "frac": 28.0 * n_elems * steps / fused_elapsed / 1e9 / HBM_PEAK_GBS,
+                            "traffic": cfg2_traffic.get("adamw_packed"),
                             "vs_two_kernels": (fused_elapsed / steps) / (elapsed / steps)},
     }
 
@@ -392,7 +410,9 @@ def region_result(cfg, steps: int, warmup: int, accumulate: bool = False) -> dic
     # the published peaks, moving its algorithmic bytes takes longer than its algorithmic flops
     intensity = flops[dominant] / nbytes[dominant]
     ridge = MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
-    traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name.split("-")[0], {}).get(dominant)
+    # the weight-gradient kernels that add to existing gradients have rows of their own (they read the old values)
+    in_place = accumulate and dominant.startswith("swiglu_wgrad")
+    traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name.split("-")[0], {}).get(dominant + ("_accumulate" if in_place else ""))
     if intensity < ridge:
         achieved = nbytes[dominant] / (dom["avg_ms"] * 1e-3) / 1e9
         roof = {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
