@@ -176,6 +176,27 @@ def test_assignment_equals_the_restated_reference_rule_on_random_inputs():
     assert reordered < 20000 // 4
 
 
+def test_hand_cases_pin_the_restated_rule_itself():
+    """The hand-worked cases above, put to oracle.planner.assign_buckets directly (parameter i used
+    by node i alone where the case gives no use ranges), so that the checker does not rest on its
+    agreement with the product alone."""
+    from oracle.planner import assign_buckets
+
+    def members(sizes, ranges, limit):
+        ranges = ranges if ranges is not None else [(i, i) for i in range(len(sizes))]
+        return [sorted(m) for _, _, m in assign_buckets(sizes, ranges, limit)]
+
+    assert members([10, 10, 10, 10], None, 25) == [[0, 1], [2, 3]]
+    assert members([30, 5, 5], None, 25) == [[0], [1, 2]]
+    assert members([10, 15, 1], None, 25) == [[0, 1], [2]]
+    assert members([20, 20], [(0, 2), (1, 3)], 25) == [[0, 1]]
+    assert members([20, 20], [(5, 6), (0, 1)], 25) == [[1], [0]]
+    assert members([10, 10, 10, 10], [(0, 0), (1, 3), (2, 6), (5, 5)], 20) == [[0, 1, 2, 3]]
+    assert members([10] * 6, [(0, 0), (1, 1), (2, 2), (3, 3), (8, 8), (9, 9)], 20) == [[0, 1], [2, 3], [4, 5]]
+    spans = [(f, l) for f, l, _ in assign_buckets([20, 20], [(0, 2), (1, 3)], 25)]
+    assert spans == [(0, 3)]
+
+
 def test_bucket_size_of_a_schedule_cuts_the_stage():
     """replicate.bucket_size (MB) -> bytes per stage -> node groups -> bucket ids for device_tasks."""
     from piper_amd.schedule import device_tasks, plan_stage_buckets, stage_bucket_bytes
