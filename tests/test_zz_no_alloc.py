@@ -58,12 +58,18 @@ def test_static_sort_matches_workspace_sort_twice_in_a_row(dev):
     out = _run_both(big, E, dev)
     assert out["counts"][17].item() == 0 and out["starts"][E].item() == big.numel()
     # second call, smaller and ragged (not a multiple of the 512-slot chunk), fewer experts
+    mid = torch.randint(0, 120, (60003,), generator=g, dtype=torch.int32).to(dev)
+    print("[case] static sort A=60003 E=120", flush=True)
+    out = _run_both(mid, 120, dev)
+    assert out["starts"][120].item() == mid.numel()
+    import numpy as np
+    assert np.array_equal(out["perm"].cpu().numpy(), np.argsort(mid.cpu().numpy(), kind="stable").astype(np.int32))
+    # third call: a short input
     small = torch.randint(0, 8, (1000 * 2 + 3,), generator=g, dtype=torch.int32).to(dev)
     print("[case] static sort A=2003 E=8", flush=True)
     out = _run_both(small, 8, dev)
     assert out["starts"][8].item() == small.numel()
-    # oracle for the second call: numpy's stable argsort
-    import numpy as np
+    # oracle for the third call: numpy's stable argsort
     ref_perm = np.argsort(small.cpu().numpy(), kind="stable").astype(np.int32)
     assert np.array_equal(out["perm"].cpu().numpy(), ref_perm)
 
@@ -98,7 +104,7 @@ def test_static_sort_recorded_into_a_hip_graph(dev):
     lib = _lib.load()
     _lib.init_device()
     g = torch.Generator().manual_seed(3)
-    shapes = [(4096 * 8, 128), (1000 * 2 + 3, 8)]
+    shapes = [(8192 * 8, 128), (1000 * 2 + 3, 8)]
     inputs = [torch.zeros(A, dtype=torch.int32, device=dev) for A, _ in shapes]
     outs = [_outputs(A, E, dev) for A, E in shapes]
 
