@@ -10,8 +10,10 @@
 // and turned into MFMA fragments by the transposing LDS read (ds_read_b64_tr_b16).
 // An fp32 operand can also be handed over already split (split3_t: three bf16 planes in memory, made
 // once by split_planes_kernel): every workgroup that loads a tile of an fp32 operand otherwise
-// splits it again, and with tiles this small that arithmetic (about 20 vector instructions per
-// MFMA) is what the kernels spend most of their time on.
+// splits it again (about 20 vector instructions per MFMA with tiles this small).  The planes are
+// 6 bytes per element where the fp32 value is 4, so this pays only where the split arithmetic is
+// what the kernel waits for: measured, the gate weight gradient (a long reduction over the tokens,
+// d_logits re-read by every column tile) gains a fifth, the forward and the d_x GEMM lose.
 #pragma once
 #include "mfma_f32_gemm.h"
 #include <type_traits>
