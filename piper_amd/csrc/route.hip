@@ -186,9 +186,17 @@ __global__ __launch_bounds__(1024) void sort_scan_kernel(int32_t* __restrict__ c
   const int e = threadIdx.x % epad, g = threadIdx.x / epad;
   const int cpg = (nchunks + G - 1) / G;
   const int c0 = g * cpg, c1 = min(nchunks, c0 + cpg);
+  // (both walks over the chunks fetch eight values at a time: one round trip per eight chunks)
+  constexpr int WALK = 8;
   int mine = 0;
   if (e < E)
-    for (int c = c0; c < c1; ++c) mine += chunk_hist[(int64_t)c * E + e];
+    for (int c = c0; c < c1; c += WALK) {
+      int v[WALK];
+#pragma unroll
+      for (int i = 0; i < WALK; ++i) v[i] = c + i < c1 ? chunk_hist[(int64_t)(c + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < WALK; ++i) mine += v[i];
+    }
   part[threadIdx.x] = mine;
   __syncthreads();
   int total = 0, before = 0;      // rows of expert e in all chunks / in the chunks of earlier groups
@@ -227,10 +235,16 @@ __global__ __launch_bounds__(1024) void sort_scan_kernel(int32_t* __restrict__ c
       if (e == E - 1) starts[E] = scan[e];
     }
     int run = start + before;
-    for (int c = c0; c < c1; ++c) {
-      const int v = chunk_hist[(int64_t)c * E + e];
-      chunk_hist[(int64_t)c * E + e] = run;
-      run += v;
+    for (int c = c0; c < c1; c += WALK) {
+      int v[WALK];
+#pragma unroll
+      for (int i = 0; i < WALK; ++i) v[i] = c + i < c1 ? chunk_hist[(int64_t)(c + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < WALK; ++i)
+        if (c + i < c1) {
+          chunk_hist[(int64_t)(c + i) * E + e] = run;
+          run += v[i];
+        }
     }
   }
 }
